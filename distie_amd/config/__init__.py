@@ -3,11 +3,12 @@ from .model_config import (ConfigError, LayerCall, LayerSpec, ModelSpec, PartSpe
                            read_config_json)
 from .duparax_config import DuparaxConfig
 from .musutar_config import MusutarConfig
+from .sekazen_config import SekazenConfig
 from .registry import (architecture_of, config_from_dict, known_architectures, load_model_config,
                        model_spec_from_dir, register_architecture)
 
 __all__ = [
     "EngineConfig", "resolve_dtype", "ConfigError", "LayerCall", "LayerSpec", "ModelSpec", "PartSpec",
-    "Qwen2Config", "MusutarConfig", "DuparaxConfig", "read_config_json", "architecture_of", "config_from_dict", "known_architectures",
+    "Qwen2Config", "MusutarConfig", "DuparaxConfig", "SekazenConfig", "read_config_json", "architecture_of", "config_from_dict", "known_architectures",
     "load_model_config", "model_spec_from_dir", "register_architecture",
 ]

@@ -13,6 +13,7 @@ from typing import Any, Dict, Mapping
 from .model_config import ConfigError, ModelSpec, Qwen2Config, read_config_json
 from .duparax_config import DuparaxConfig
 from .musutar_config import MusutarConfig
+from .sekazen_config import SekazenConfig
 
 _ARCHITECTURES: Dict[str, Any] = {}
 
@@ -71,3 +72,4 @@ def model_spec_from_dir(model_dir) -> ModelSpec:
 register_architecture(Qwen2Config.architecture, Qwen2Config)
 register_architecture(MusutarConfig.architecture, MusutarConfig)
 register_architecture(DuparaxConfig.architecture, DuparaxConfig)
+register_architecture(SekazenConfig.architecture, SekazenConfig)

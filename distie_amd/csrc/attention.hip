@@ -94,7 +94,8 @@ __global__ __launch_bounds__(DISTIE_WAVE * WAVES) void attn_generic_kernel(
     const T* __restrict__ qkv, int64_t q_stride, const C* __restrict__ k_cache, const C* __restrict__ v_cache,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ token_request,
     const int32_t* __restrict__ block_table, int table_width, const int32_t* __restrict__ table_rows, T* __restrict__ out, int heads, int kv_heads,
-    int block_size, float scale, int window, const float* __restrict__ head_slopes, float score_cap) {
+    int block_size, float scale, int window, const float* __restrict__ head_slopes, float score_cap,
+    const float* __restrict__ sinks) {
   __shared__ float q_s[D];
   __shared__ float p_s[WAVES][DISTIE_WAVE];
   __shared__ int64_t base_s[WAVES][DISTIE_WAVE];
@@ -175,8 +176,12 @@ __global__ __launch_bounds__(DISTIE_WAVE * WAVES) void attn_generic_kernel(
     }
   }
   T* o = out + (t * heads + h) * D;
+  // a sink joins the denominator as exp(sink), once, with no value: as one more maximum and one more term of the sum
+  const float sink = sinks != nullptr ? sinks[h] : -INFINITY;
   if constexpr (WAVES == 1) {
-    const float inv = 1.f / l;
+    const float top = fmaxf(m, sink);
+    const float weight = expf(m - top);
+    const float inv = weight / (l * weight + expf(sink - top));
 #pragma unroll
     for (int i = 0; i < DIMS_PER_LANE; ++i) {
       const int d = lane + i * DISTIE_WAVE;
@@ -194,9 +199,9 @@ __global__ __launch_bounds__(DISTIE_WAVE * WAVES) void attn_generic_kernel(
     }
     __syncthreads();
     if (wave != 0) return;
-    float top = -INFINITY;
+    float top = sink;
     for (int w = 0; w < WAVES; ++w) top = fmaxf(top, m_s[w]);
-    float total = 0.f;
+    float total = sink == -INFINITY ? 0.f : expf(sink - top);
     float weight[WAVES];
     for (int w = 0; w < WAVES; ++w) {
       weight[w] = m_s[w] == -INFINITY ? 0.f : expf(m_s[w] - top);       // a wave without keys counts nothing
@@ -228,7 +233,8 @@ __global__ __launch_bounds__(DISTIE_WAVE * WAVES) void attn_grouped_f32_kernel(
     const float* __restrict__ qkv, int64_t q_stride, const float* __restrict__ k_cache, const float* __restrict__ v_cache,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ token_request,
     const int32_t* __restrict__ block_table, int table_width, const int32_t* __restrict__ table_rows,
-    float* __restrict__ out, int heads, int kv_heads, int parts, int block_size, float scale, int window) {
+    float* __restrict__ out, int heads, int kv_heads, int parts, int block_size, float scale, int window,
+    const float* __restrict__ sinks) {
   __shared__ float p_s[WAVES][G][DISTIE_WAVE];
   __shared__ int64_t base_s[WAVES][DISTIE_WAVE];
   __shared__ float m_s[WAVES][G], l_s[WAVES][G];
@@ -393,9 +399,10 @@ __global__ __launch_bounds__(DISTIE_WAVE * WAVES) void attn_grouped_f32_kernel(
   __syncthreads();
   // wave w writes heads w, w + WAVES, ... of the part
   for (int g = wave; g < n; g += WAVES) {
-    float top = -INFINITY;
+    const float sink = sinks != nullptr ? sinks[h0 + g] : -INFINITY;      // one more term of the denominator, no value
+    float top = sink;
     for (int w = 0; w < WAVES; ++w) top = fmaxf(top, m_s[w][g]);
-    float total = 0.f;
+    float total = sink == -INFINITY ? 0.f : expf(sink - top);
     float weight[WAVES];
     for (int w = 0; w < WAVES; ++w) {
       weight[w] = m_s[w][g] == -INFINITY ? 0.f : expf(m_s[w][g] - top);    // a wave without keys counts nothing
@@ -416,13 +423,14 @@ __global__ __launch_bounds__(DISTIE_WAVE * WAVES) void attn_grouped_f32_kernel(
 
 // qkv: [T, q_stride] with q of head h at columns h*D; out: [T, heads*D]. window = 0: every earlier key.
 // head_slopes (float32 [heads], may be null): score += slope[h] * (key - position); score_cap > 0: the scaled score
-// goes through cap * tanh(score / cap) first. Only this kernel takes the two.
+// goes through cap * tanh(score / cap) first. Only this kernel takes the two. sinks (float32 [heads], may be null): the
+// softmax's denominator holds exp(sinks[h]) beside the keys' terms; every kernel of this file takes them.
 extern "C" int distie_attention_generic(const void* qkv, int dtype, int64_t q_stride, const void* k_cache,
                                         const void* v_cache, int cache_dtype, const int32_t* positions,
                                         const int32_t* token_request, const int32_t* block_table,
                                         int table_width, const int32_t* table_rows, void* out, int tokens, int heads, int kv_heads,
                                         int block_size, float scale, int window, const float* head_slopes,
-                                        float score_cap, hipStream_t stream) {
+                                        float score_cap, const float* sinks, hipStream_t stream) {
   if (tokens <= 0) return 0;
   if (heads < 1 || kv_heads < 1 || heads % kv_heads != 0 || block_size < 1 || table_width < 1 || window < 0 ||
       score_cap < 0.f)
@@ -443,7 +451,7 @@ extern "C" int distie_attention_generic(const void* qkv, int dtype, int64_t q_st
     attn_grouped_f32_kernel<G, WAVES><<<grouped, DISTIE_WAVE * WAVES, 0, stream>>>(                                  \
         static_cast<const float*>(qkv), q_stride, static_cast<const float*>(k_cache),                               \
         static_cast<const float*>(v_cache), positions, token_request, block_table, table_width, table_rows,         \
-        static_cast<float*>(out), heads, kv_heads, parts, block_size, scale, window)
+        static_cast<float*>(out), heads, kv_heads, parts, block_size, scale, window, sinks)
     if (per == 4) DISTIE_GROUPED(4, 8);
     else if (per == 2) DISTIE_GROUPED(2, 8);
     else DISTIE_GROUPED(1, 8);
@@ -456,13 +464,13 @@ extern "C" int distie_attention_generic(const void* qkv, int dtype, int64_t q_st
         (attn_generic_kernel<T, C, 8><<<grid, DISTIE_WAVE * 8, 0, stream>>>(
             static_cast<const T*>(qkv), q_stride, static_cast<const C*>(k_cache), static_cast<const C*>(v_cache),
             positions, token_request, block_table, table_width, table_rows, static_cast<T*>(out), heads, kv_heads, block_size,
-            scale, window, head_slopes, score_cap))));
+            scale, window, head_slopes, score_cap, sinks))));
   } else {
     DISTIE_DISPATCH(dtype, T, DISTIE_DISPATCH(cache_dtype, C,
         (attn_generic_kernel<T, C, 1><<<grid, DISTIE_WAVE, 0, stream>>>(
             static_cast<const T*>(qkv), q_stride, static_cast<const C*>(k_cache), static_cast<const C*>(v_cache),
             positions, token_request, block_table, table_width, table_rows, static_cast<T*>(out), heads, kv_heads, block_size,
-            scale, window, head_slopes, score_cap))));
+            scale, window, head_slopes, score_cap, sinks))));
   }
   return launch_status();
 }
@@ -500,6 +508,16 @@ constexpr bool DK_TAIL = (D % 32) != 0; // one more step of 16
 constexpr int DB16 = D / 16;            // 16-wide blocks of the output
 constexpr int DC_BLOCKS = (D <= 128) ? 4 : 2;   // blocks of 16 keys whose loads are in flight together
 constexpr int DC_KEYS = 16 * DC_BLOCKS;
+
+// What a sink does to a finished column: with the keys' maximum m and sum l (in units of log 2, l relative to m) and the
+// sink z (the same units; -inf: none), the factor on the unnormalised output is 2^(m - top) / (l 2^(m - top) + 2^(z - top)),
+// top = max(m, z): exp(z) is one more term of the denominator and has no value.
+__device__ __forceinline__ float sink_factor(float m, float l, float sink2) {
+  if (sink2 == -INFINITY) return 1.f / l;
+  const float top = fmaxf(m, sink2);
+  const float weight = m == -INFINITY ? 0.f : fast_exp2(m - top);
+  return weight / (l * weight + fast_exp2(sink2 - top));
+}
 
 // How one request's keys are cut into runs. The visible keys (all of them, or the window's), counted from the
 // 64-key boundary at or before the first of them, are cut into at most `max_splits` runs of one length, a
@@ -799,7 +817,7 @@ template <bool FAST>
 __global__ __launch_bounds__(RD_THREADS) void attn_reduce_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml, const int32_t* __restrict__ kv_len,
     const int32_t* __restrict__ cu_q, bf16_t* __restrict__ out, int heads, int window, int max_splits,
-    int dense_rows, const int32_t* __restrict__ shared_run_len) {
+    int dense_rows, const int32_t* __restrict__ shared_run_len, const float* __restrict__ sinks) {
   __shared__ float weight_s[FAST ? RD_FAST_RUNS : RD_MAX_RUNS];
   __shared__ float sum_s[RD_WAVES][D];
   __shared__ float scratch[32];
@@ -831,6 +849,8 @@ __global__ __launch_bounds__(RD_THREADS) void attn_reduce_kernel(
   const int runs = key_runs(q_pos, window, max_splits, shared_run_len != nullptr ? *shared_run_len : 0).count;     // the first `runs` places hold results
   const int64_t base = base0;
   bf16_t* o = out + (static_cast<int64_t>(token) * heads + head) * D;
+  // a sink: one more maximum and one more term of the denominator, in the runs' units of log 2; it has no value
+  const float sink = sinks != nullptr ? sinks[head] * 1.4426950408889634f : -INFINITY;
 
   if constexpr (FAST) {
     const bool mine = tid < runs;
@@ -838,10 +858,11 @@ __global__ __launch_bounds__(RD_THREADS) void attn_reduce_kernel(
     m = wave_max(m);
     if (lane == 0) scratch[wave] = m;
     __syncthreads();
-    m = fmaxf(fmaxf(scratch[0], scratch[1]), fmaxf(scratch[2], scratch[3]));
+    m = fmaxf(fmaxf(fmaxf(scratch[0], scratch[1]), fmaxf(scratch[2], scratch[3])), sink);
     const float w = mine ? fast_exp2(early_ml.x - m) : 0.f;
     if (tid < RD_FAST_RUNS) weight_s[tid] = w;
-    const float l = block_sum(mine ? w * early_ml.y : 0.f, scratch + 16);     // has the barrier that publishes the weights
+    const float l = block_sum(mine ? w * early_ml.y : 0.f, scratch + 16) +     // has the barrier that publishes the weights
+                    (sink == -INFINITY ? 0.f : fast_exp2(sink - m));
 #pragma unroll
     for (int i = 0; i < DIMS_PER_LANE; ++i) {
       const int d = lane + i * DISTIE_WAVE;
@@ -872,7 +893,7 @@ __global__ __launch_bounds__(RD_THREADS) void attn_reduce_kernel(
   m = wave_max(m);
   if (lane == 0) scratch[wave] = m;
   __syncthreads();
-  m = fmaxf(fmaxf(scratch[0], scratch[1]), fmaxf(scratch[2], scratch[3]));
+  m = fmaxf(fmaxf(fmaxf(scratch[0], scratch[1]), fmaxf(scratch[2], scratch[3])), sink);
   float l = 0.f;
   for (int j = tid; j < runs; j += RD_THREADS) {
     const float w = fast_exp2(part_ml[2 * (base + j)] - m);
@@ -880,6 +901,7 @@ __global__ __launch_bounds__(RD_THREADS) void attn_reduce_kernel(
     l += w * part_ml[2 * (base + j) + 1];
   }
   l = block_sum(l, scratch + 16);           // has the barrier that publishes the weights
+  if (sink != -INFINITY) l += fast_exp2(sink - m);
   const float* po = part_o + base * D;
 #pragma unroll
   for (int i = 0; i < DIMS_PER_LANE; ++i) {
@@ -924,7 +946,7 @@ extern "C" int distie_attention_decode_bf16(const void* qkv, int64_t q_stride, c
                                             int table_width, const int32_t* table_rows, void* out, float* part_o, float* part_ml,
                                             int num_requests, int heads, int kv_heads, int block_size, float scale,
                                             int window, int split_hint, int max_splits, int dense_rows,
-                                            const int32_t* shared_run_len, hipStream_t stream) {
+                                            const int32_t* shared_run_len, const float* sinks, hipStream_t stream) {
   if (num_requests <= 0) return 0;
   const int group = kv_heads > 0 ? heads / kv_heads : 0;
   if (heads < 1 || kv_heads < 1 || heads % kv_heads != 0 || block_size % 16 != 0 || table_width < 1 || window < 0 ||
@@ -952,10 +974,12 @@ extern "C" int distie_attention_decode_bf16(const void* qkv, int64_t q_stride, c
   if (status != 0) return status;
   if (max_splits <= RD_FAST_RUNS) {
     attn_reduce_kernel<true><<<dim3(heads, num_requests), RD_THREADS, 0, stream>>>(
-        part_o, part_ml, kv_len, cu_q, static_cast<bf16_t*>(out), heads, window, max_splits, dense_rows, shared_run_len);
+        part_o, part_ml, kv_len, cu_q, static_cast<bf16_t*>(out), heads, window, max_splits, dense_rows, shared_run_len,
+        sinks);
   } else {
     attn_reduce_kernel<false><<<dim3(heads, num_requests), RD_THREADS, 0, stream>>>(
-        part_o, part_ml, kv_len, cu_q, static_cast<bf16_t*>(out), heads, window, max_splits, dense_rows, shared_run_len);
+        part_o, part_ml, kv_len, cu_q, static_cast<bf16_t*>(out), heads, window, max_splits, dense_rows, shared_run_len,
+        sinks);
   }
   return launch_status();
 }
@@ -1005,7 +1029,7 @@ __global__ __launch_bounds__(PF_THREADS, (D <= 128) ? 2 : 1) void attn_prefill_k
     const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ positions, const int32_t* __restrict__ cu_q,
     const int32_t* __restrict__ block_table, int table_width, const int32_t* __restrict__ table_rows, bf16_t* __restrict__ out, float* __restrict__ part_o,
     float* __restrict__ part_ml, int tokens, int num_requests, int heads, int kv_heads, int block_size, float scale,
-    int window, int min_q_len) {
+    int window, int min_q_len, const float* __restrict__ sinks) {
   __shared__ __attribute__((aligned(16))) bf16_t k_lds[PF_BN * PF_K_STRIDE];
   __shared__ __attribute__((aligned(16))) bf16_t v_lds[32 * PF_DB * PF_V_STRIDE];
   const int tid = threadIdx.x;
@@ -1258,7 +1282,7 @@ __global__ __launch_bounds__(PF_THREADS, (D <= 128) ? 2 : 1) void attn_prefill_k
   const int64_t row = static_cast<int64_t>(token0 + wave_col0 + c) * heads + head;
   if (gridDim.z == 1) {
     bf16_t* o = out + row * D;
-    const float inv = 1.f / l_run;
+    const float inv = sink_factor(m_run, l_run, sinks != nullptr ? sinks[head] * 1.4426950408889634f : -INFINITY);
 #pragma unroll
     for (int db = 0; db < PF_DB; ++db)
 #pragma unroll
@@ -1296,7 +1320,8 @@ constexpr int PF_MAX_SPLITS = 16;
 template <typename OUT, int MOST>
 __global__ void attn_prefill_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                           const int32_t* __restrict__ token_request, const int32_t* __restrict__ cu_q,
-                                          OUT* __restrict__ out, int tokens, int heads, int min_q_len, int splits) {
+                                          OUT* __restrict__ out, int tokens, int heads, int min_q_len, int splits,
+                                          const float* __restrict__ sinks) {
   const int64_t token = blockIdx.x;
   const int request = token_request[token];
   if (cu_q[request + 1] - cu_q[request] < min_q_len) return;
@@ -1322,7 +1347,10 @@ __global__ void attn_prefill_merge_kernel(const float* __restrict__ part_o, cons
         m = fmaxf(m, ml[s].x);
       }
     }
-    float l = 0.f;
+    // a sink: one more maximum and one more term of the denominator, without a value
+    const float sink = sinks != nullptr ? sinks[head] * 1.4426950408889634f : -INFINITY;
+    m = fmaxf(m, sink);
+    float l = sink == -INFINITY ? 0.f : fast_exp2(sink - m);
     float4 sum = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int s = 0; s < MOST; ++s) {
@@ -1350,18 +1378,19 @@ __global__ void attn_prefill_merge_kernel(const float* __restrict__ part_o, cons
 // so that few parts leave room for more waves on a compute unit.
 template <typename OUT>
 static void launch_merge(const float* part_o, const float* part_ml, const int32_t* token_request, const int32_t* cu_q,
-                         OUT* out, int tokens, int heads, int min_q_len, int splits, hipStream_t stream) {
+                         OUT* out, int tokens, int heads, int min_q_len, int splits, const float* sinks,
+                         hipStream_t stream) {
   const int work = heads * (D / 4);
   const int threads = work >= 512 ? 512 : (work >= 256 ? 256 : 64);
   if (splits <= 4)
     attn_prefill_merge_kernel<OUT, 4><<<tokens, threads, 0, stream>>>(part_o, part_ml, token_request, cu_q, out, tokens,
-                                                                       heads, min_q_len, splits);
+                                                                       heads, min_q_len, splits, sinks);
   else if (splits <= 8)
     attn_prefill_merge_kernel<OUT, 8><<<tokens, threads, 0, stream>>>(part_o, part_ml, token_request, cu_q, out, tokens,
-                                                                       heads, min_q_len, splits);
+                                                                       heads, min_q_len, splits, sinks);
   else
     attn_prefill_merge_kernel<OUT, PF_MAX_SPLITS><<<tokens, threads, 0, stream>>>(part_o, part_ml, token_request, cu_q, out,
-                                                                                   tokens, heads, min_q_len, splits);
+                                                                                   tokens, heads, min_q_len, splits, sinks);
 }
 
 // Portions of prompts (and whole mixed steps). bfloat16 only; block_size must be a multiple of 16. Requests that
@@ -1371,7 +1400,7 @@ extern "C" int distie_attention_prefill_bf16(const void* qkv, int64_t q_stride, 
                                              int table_width, const int32_t* table_rows, void* out, int tokens, int num_requests, int heads,
                                              int kv_heads, int block_size, float scale, int window, int min_q_len,
                                              const int32_t* token_request, float* part_o, float* part_ml,
-                                             int splits, hipStream_t stream) {
+                                             int splits, const float* sinks, hipStream_t stream) {
   // splits > 1: the keys are walked in that many parts side by side (worth it for long portions), with
   // part_o (float32 [splits, tokens, heads, D]) and part_ml (float32 [splits, tokens, heads, 2]) in between.
   if (tokens <= 0) return 0;
@@ -1384,10 +1413,10 @@ extern "C" int distie_attention_prefill_bf16(const void* qkv, int64_t q_stride, 
   attn_prefill_kernel<<<dim3(heads, tiles, splits), PF_THREADS, 0, stream>>>(
       static_cast<const bf16_t*>(qkv), q_stride, static_cast<const bf16_t*>(k_cache), static_cast<const bf16_t*>(v_cache),
       positions, cu_q, block_table, table_width, table_rows, static_cast<bf16_t*>(out), part_o, part_ml, tokens, num_requests, heads,
-      kv_heads, block_size, scale, window, min_q_len);
+      kv_heads, block_size, scale, window, min_q_len, sinks);
   int status = launch_status();
   if (status != 0 || splits == 1) return status;
-  launch_merge(part_o, part_ml, token_request, cu_q, static_cast<bf16_t*>(out), tokens, heads, min_q_len, splits, stream);
+  launch_merge(part_o, part_ml, token_request, cu_q, static_cast<bf16_t*>(out), tokens, heads, min_q_len, splits, sinks, stream);
   return launch_status();
 }
 
@@ -1413,7 +1442,7 @@ __global__ __launch_bounds__(PF_THREADS, 1) void attn_prefill_f32_kernel(
     const float* __restrict__ v_cache, const int32_t* __restrict__ positions, const int32_t* __restrict__ cu_q,
     const int32_t* __restrict__ block_table, int table_width, const int32_t* __restrict__ table_rows, float* __restrict__ out,
     float* __restrict__ part_o, float* __restrict__ part_ml, int tokens, int num_requests, int heads, int kv_heads,
-    int block_size, float scale, int window, int min_q_len) {
+    int block_size, float scale, int window, int min_q_len, const float* __restrict__ sinks) {
   __shared__ __attribute__((aligned(16))) float k_lds[PF_BN * PF32_K_STRIDE];
   __shared__ __attribute__((aligned(16))) float v_lds[D * PF32_V_STRIDE];
   const int tid = threadIdx.x;
@@ -1635,7 +1664,8 @@ __global__ __launch_bounds__(PF_THREADS, 1) void attn_prefill_f32_kernel(
   const bool whole = gridDim.z == 1;
   const int64_t at = whole ? row : static_cast<int64_t>(blockIdx.z) * tokens * heads + row;
   float* o = (whole ? out : part_o) + at * D;
-  const float factor = whole ? 1.f / l_run : 1.f;         // a part without a key for this column leaves l = 0: not read
+  // (a part without a key for this column leaves l = 0: not read)
+  const float factor = whole ? sink_factor(m_run, l_run, sinks != nullptr ? sinks[head] * 1.4426950408889634f : -INFINITY) : 1.f;
 #pragma unroll
   for (int db = 0; db < D / 32; ++db)
 #pragma unroll
@@ -1658,7 +1688,7 @@ extern "C" int distie_attention_prefill_f32(const void* qkv, int64_t q_stride, c
                                             int table_width, const int32_t* table_rows, void* out, int tokens, int num_requests, int heads,
                                             int kv_heads, int block_size, float scale, int window, int min_q_len,
                                             const int32_t* token_request, float* part_o, float* part_ml,
-                                            int splits, hipStream_t stream) {
+                                            int splits, const float* sinks, hipStream_t stream) {
 #if (DISTIE_HEAD_DIM % 32 == 0) && (DISTIE_HEAD_DIM <= 128)
   if (tokens <= 0) return 0;
   if (heads < 1 || kv_heads < 1 || heads % kv_heads != 0 || block_size % 16 != 0 || table_width < 1 || window < 0 ||
@@ -1671,10 +1701,10 @@ extern "C" int distie_attention_prefill_f32(const void* qkv, int64_t q_stride, c
   attn_prefill_f32_kernel<<<dim3(heads, tiles, splits), PF_THREADS, 0, stream>>>(
       static_cast<const float*>(qkv), q_stride, static_cast<const float*>(k_cache), static_cast<const float*>(v_cache),
       positions, cu_q, block_table, table_width, table_rows, static_cast<float*>(out), part_o, part_ml, tokens, num_requests,
-      heads, kv_heads, block_size, scale, window, min_q_len);
+      heads, kv_heads, block_size, scale, window, min_q_len, sinks);
   int status = launch_status();
   if (status != 0 || splits == 1) return status;
-  launch_merge(part_o, part_ml, token_request, cu_q, static_cast<float*>(out), tokens, heads, min_q_len, splits, stream);
+  launch_merge(part_o, part_ml, token_request, cu_q, static_cast<float*>(out), tokens, heads, min_q_len, splits, sinks, stream);
   return launch_status();
 #else
   return DISTIE_BAD_ARGUMENT;
@@ -1687,7 +1717,7 @@ extern "C" int distie_attention_decode_columns() { return 0; }
 
 extern "C" int distie_attention_decode_bf16(const void*, int64_t, const void*, const void*, const int32_t*, const int32_t*,
                                             const int32_t*, int, const int32_t*, void*, void*, void*, int, int, int, int, float, int, int,
-                                            int, int, const int32_t*, hipStream_t) {
+                                            int, int, const int32_t*, const float*, hipStream_t) {
   return DISTIE_BAD_ARGUMENT;
 }
 
@@ -1695,7 +1725,7 @@ extern "C" int distie_attention_decode_run_len(const int32_t*, int, int, int, in
 
 extern "C" int distie_attention_prefill_bf16(const void*, int64_t, const void*, const void*, const int32_t*, const int32_t*,
                                              const int32_t*, int, const int32_t*, void*, int, int, int, int, int, float, int, int,
-                                             const int32_t*, void*, void*, int, hipStream_t) {
+                                             const int32_t*, void*, void*, int, const float*, hipStream_t) {
   return DISTIE_BAD_ARGUMENT;
 }
 
@@ -1703,7 +1733,7 @@ extern "C" int distie_attention_prefill_f32_fits() { return 0; }
 
 extern "C" int distie_attention_prefill_f32(const void*, int64_t, const void*, const void*, const int32_t*, const int32_t*,
                                             const int32_t*, int, const int32_t*, void*, int, int, int, int, int, float, int, int,
-                                            const int32_t*, void*, void*, int, hipStream_t) {
+                                            const int32_t*, void*, void*, int, const float*, hipStream_t) {
   return DISTIE_BAD_ARGUMENT;
 }
 

@@ -187,7 +187,16 @@ __global__ void norm_chain_kernel(const A* __restrict__ t0, int slices0, int64_t
       store_values<V>(y_out + base + c, y);
     }
   }
-  if (residual == nullptr || pre_w == nullptr) return;
+  if (residual == nullptr || out == nullptr) return;
+  if (pre_w == nullptr) {
+    // no norm in front of the next sub-layer: it reads the new residual itself, in its own precision
+    for (int c = V * threadIdx.x; c < C; c += step) {
+      float x[V];
+      load_values<V>(row + c, x);
+      store_values<V>(out + base + c, x);
+    }
+    return;
+  }
   const float rn = 1.f / sqrtf(block_sum(q2, scratch) / C + pre_eps);
   for (int c = V * threadIdx.x; c < C; c += step) {
     float x[V], w[V];
@@ -743,10 +752,22 @@ __global__ void lru_chunk_apply_kernel(const float* __restrict__ a, const float*
 constexpr int ROUTE_MAX_EXPERTS = 1024;
 constexpr int ROUTE_MAX_TOP = 32;
 
+// the weights of the chosen experts from their logits (largest first): softmax over those alone, or each one's own sigmoid
+__device__ __forceinline__ void write_route_weights(const float* chosen, float* __restrict__ out, int top, int sigmoid) {
+  if (sigmoid) {
+    for (int k = 0; k < top; ++k) out[k] = 1.f / (1.f + expf(-chosen[k]));
+    return;
+  }
+  const float peak = chosen[0];
+  float total = 0.f;
+  for (int k = 0; k < top; ++k) total += expf(chosen[k] - peak);
+  for (int k = 0; k < top; ++k) out[k] = expf(chosen[k] - peak) / total;
+}
+
 template <typename X, typename W>
 __global__ void __launch_bounds__(256)
 route_topk_kernel(const X* __restrict__ x, const W* __restrict__ weight, const float* __restrict__ bias,
-                  int32_t* __restrict__ experts, float* __restrict__ gates, int C, int E, int top) {
+                  int32_t* __restrict__ experts, float* __restrict__ gates, int C, int E, int top, int sigmoid) {
   extern __shared__ float xs[];                       // the token's row as float32
   __shared__ float z[ROUTE_MAX_EXPERTS];
   __shared__ float chosen[ROUTE_MAX_TOP];
@@ -791,12 +812,7 @@ route_topk_kernel(const X* __restrict__ x, const W* __restrict__ weight, const f
     }
     if (at % 64 == lane) z[at] = -INFINITY;           // the lane that reads this place takes it out itself
   }
-  if (lane == 0) {
-    const float peak = chosen[0];
-    float total = 0.f;
-    for (int k = 0; k < top; ++k) total += expf(chosen[k] - peak);
-    for (int k = 0; k < top; ++k) gates[t * top + k] = expf(chosen[k] - peak) / total;
-  }
+  if (lane == 0) write_route_weights(chosen, gates + t * top, top, sigmoid);
 }
 
 // The same for bfloat16 rows and weights whose width is a multiple of 8: a thread takes 16-byte pieces of the token's
@@ -815,7 +831,7 @@ __device__ __forceinline__ void unpack8(const uint4& raw, float v[8]) {
 
 __global__ void __launch_bounds__(256)
 route_topk_bf16_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ weight, const float* __restrict__ bias,
-                       int32_t* __restrict__ experts, float* __restrict__ gates, int C, int E, int top) {
+                       int32_t* __restrict__ experts, float* __restrict__ gates, int C, int E, int top, int sigmoid) {
   __shared__ float z[ROUTE_MAX_EXPERTS];
   __shared__ float part[4][ROUTE_GROUP];
   __shared__ float chosen[ROUTE_MAX_TOP];
@@ -874,12 +890,7 @@ route_topk_bf16_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ 
     }
     if (at % 64 == lane) z[at] = -INFINITY;
   }
-  if (lane == 0) {
-    const float peak = chosen[0];
-    float total = 0.f;
-    for (int k = 0; k < top; ++k) total += expf(chosen[k] - peak);
-    for (int k = 0; k < top; ++k) gates[t * top + k] = expf(chosen[k] - peak) / total;
-  }
+  if (lane == 0) write_route_weights(chosen, gates + t * top, top, sigmoid);
 }
 
 // hidden [T, ld]: the columns [e * F, (e + 1) * F) of expert e times the row's weight for e, zero if e was not chosen
@@ -920,6 +931,51 @@ __global__ void route_scale_bf16x8_kernel(bf16_t* __restrict__ hidden, int64_t l
              (static_cast<uint32_t>(__builtin_bit_cast(uint16_t, static_cast<bf16_t>(v[2 * k + 1] * g))) << 16);
     *p = uint4{w[0], w[1], w[2], w[3]};
   }
+}
+
+// The hidden values of routed gated experts from the stacked product: gate_up [T, ld] holds every expert's gate columns
+// (E x F), then every expert's up columns; `slices` partial sums lie `stride` elements apart. For the expert e that owns
+// column c, chosen by the row with weight w: g and u times w if `on_input`, clamped if limit > 0 (g from above, u on both
+// sides), hidden = g * sigmoid(slope * g) * (u + up_shift), times w unless `on_input`; zero if the row did not choose e.
+// V columns a thread (V > 1: F a multiple of V, 16-byte aligned rows).
+template <int V, typename X, typename O>
+__global__ void route_glu_kernel(const X* __restrict__ gate_up, int64_t ld, int slices, int64_t stride,
+                                 const int32_t* __restrict__ experts, const float* __restrict__ gates, int top, int F,
+                                 int width, float limit, float slope, float up_shift, int on_input, O* __restrict__ out,
+                                 int64_t T) {
+  const int pieces = width / V;
+  const int64_t total = T * pieces;
+  for (int64_t it = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; it < total;
+       it += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+    const int64_t t = it / pieces;
+    const int c = V * static_cast<int>(it % pieces);
+    const int e = c / F;
+    float w = 0.f;
+    bool chosen = false;
+    for (int k = 0; k < top; ++k)
+      if (experts[t * top + k] == e) w = gates[t * top + k], chosen = true;
+    float h[V] = {};
+    if (chosen) {
+      float g[V], u[V];
+      sum_values<V>(gate_up + t * ld + c, slices, stride, g);
+      sum_values<V>(gate_up + t * ld + width + c, slices, stride, u);
+#pragma unroll
+      for (int k = 0; k < V; ++k) {
+        float gk = g[k], uk = u[k];
+        if (on_input) gk *= w, uk *= w;
+        if (limit > 0.f) gk = fminf(gk, limit), uk = fminf(fmaxf(uk, -limit), limit);
+        h[k] = gk / (1.f + expf(-slope * gk)) * (uk + up_shift);
+        if (!on_input) h[k] *= w;
+      }
+    }
+    store_values<V>(out + t * width + c, h);
+  }
+}
+
+// x <- cap * tanh(x / cap)
+__global__ void softcap_f32_kernel(float* __restrict__ x, int64_t count, float cap) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i < count) x[i] = cap * tanhf(x[i] / cap);
 }
 
 __global__ void scale_f32_kernel(float* __restrict__ x, int64_t count, float scale) {
@@ -1108,7 +1164,8 @@ extern "C" int distie_lru_scan_chunked(const float* a, const float* x, float* st
 }
 
 extern "C" int distie_route_topk(const void* x, int x_dtype, const void* weight, int w_dtype, const float* bias,
-                                 int32_t* experts, float* gates, int T, int C, int E, int top, hipStream_t stream) {
+                                 int32_t* experts, float* gates, int T, int C, int E, int top, int sigmoid,
+                                 hipStream_t stream) {
   if (T <= 0) return 0;
   if (C < 1 || E < 1 || E > ROUTE_MAX_EXPERTS || top < 1 || top > E || top > ROUTE_MAX_TOP ||
       static_cast<size_t>(C) * sizeof(float) > 96 * 1024)
@@ -1116,7 +1173,7 @@ extern "C" int distie_route_topk(const void* x, int x_dtype, const void* weight,
   if (x_dtype == DISTIE_BF16 && w_dtype == DISTIE_BF16 && C % 8 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 &&
       reinterpret_cast<uintptr_t>(weight) % 16 == 0) {
     route_topk_bf16_kernel<<<T, 256, 0, stream>>>(static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(weight), bias,
-                                                  experts, gates, C, E, top);
+                                                  experts, gates, C, E, top, sigmoid);
     return launch_status();
   }
   const size_t lds = static_cast<size_t>(C) * sizeof(float);
@@ -1126,7 +1183,7 @@ extern "C" int distie_route_topk(const void* x, int x_dtype, const void* weight,
                             hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)) != hipSuccess)
       return DISTIE_BAD_ARGUMENT;
     route_topk_kernel<X, W><<<T, 256, lds, stream>>>(static_cast<const X*>(x), static_cast<const W*>(weight), bias,
-                                                     experts, gates, C, E, top);
+                                                     experts, gates, C, E, top, sigmoid);
   }));
   return launch_status();
 }
@@ -1146,6 +1203,42 @@ extern "C" int distie_route_scale(void* hidden, int dtype, int64_t ld, const int
   const dim3 grid(T, per_row < 64 ? per_row : 64);
   DISTIE_DISPATCH(dtype, X, route_scale_kernel<X><<<grid, 256, 0, stream>>>(static_cast<X*>(hidden), ld, experts, gates,
                                                                             top, F, width));
+  return launch_status();
+}
+
+// gate_up: [T, ld] of `dtype`, or `slices` float32 partial sums [slices, T, ld]; out: [T, E * F] of `out_dtype`.
+// limit <= 0: no clamps.
+extern "C" int distie_route_glu(const void* gate_up, int dtype, int64_t ld, int slices, const int32_t* experts,
+                                const float* gates, int T, int top, int E, int F, float limit, float slope, float up_shift,
+                                int on_input, void* out, int out_dtype, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (top < 1 || E < 1 || F < 1 || slices < 1 || (slices > 1 && dtype != DISTIE_F32) || ld < 2 * static_cast<int64_t>(E) * F)
+    return DISTIE_BAD_ARGUMENT;
+  const int width = E * F;
+  const int64_t stride = static_cast<int64_t>(T) * ld;
+  const bool wide = F % 4 == 0 && ld % 4 == 0 && reinterpret_cast<uintptr_t>(gate_up) % 16 == 0 &&
+                    reinterpret_cast<uintptr_t>(out) % 16 == 0;
+  const int64_t items = static_cast<int64_t>(T) * (wide ? width / 4 : width);
+  const int blocks = static_cast<int>(items / 256 + 1 < 16384 ? items / 256 + 1 : 16384);
+#define DISTIE_ROUTE_GLU(V)                                                                                           \
+  DISTIE_DISPATCH(dtype, X, DISTIE_DISPATCH(out_dtype, O, (route_glu_kernel<V, X, O><<<blocks, 256, 0, stream>>>(     \
+      static_cast<const X*>(gate_up), ld, slices, stride, experts, gates, top, F, width, limit, slope, up_shift,      \
+      on_input, static_cast<O*>(out), T))))
+  if (wide) {
+    DISTIE_ROUTE_GLU(4);
+  } else {
+    DISTIE_ROUTE_GLU(1);
+  }
+#undef DISTIE_ROUTE_GLU
+  return launch_status();
+}
+
+extern "C" int distie_softcap_f32(float* x, int64_t count, float cap, hipStream_t stream) {
+  if (count <= 0) return 0;
+  if (!(cap > 0.f)) return DISTIE_BAD_ARGUMENT;
+  const int64_t blocks = (count + 255) / 256;
+  if (blocks > 0x7fffffff) return DISTIE_BAD_ARGUMENT;
+  softcap_f32_kernel<<<static_cast<unsigned>(blocks), 256, 0, stream>>>(x, count, cap);
   return launch_status();
 }
 

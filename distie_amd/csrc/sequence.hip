@@ -267,7 +267,8 @@ __global__ void conv_rope_kv_write_kernel(const X* __restrict__ product, int64_t
                                           const int32_t* __restrict__ cu_q, const int32_t* __restrict__ token_request,
                                           const int32_t* __restrict__ state_slots, int H, int G, int D, int E, int DP,
                                           int block_size, int has_kv, int write, const int32_t* __restrict__ positions,
-                                          float temp_coef, int temp_every) {
+                                          float temp_coef, int temp_every, const float* __restrict__ q_norm,
+                                          const float* __restrict__ k_norm, float norm_eps) {
   const int64_t t = blockIdx.x;
   const int head = blockIdx.y;
   const int N = H * D + (has_kv ? G * (D + E) : 0);
@@ -305,33 +306,48 @@ __global__ void conv_rope_kv_write_kernel(const X* __restrict__ product, int64_t
     }
     return;
   }
-  // q and k: a thread owns a pair, or a single dimension beyond the turned ones
+  // q and k: a thread owns a pair, or a single dimension beyond the turned ones (the launcher gives a block at least
+  // DP - pairs threads, so a thread has one item and the whole head is in the block at once)
   const int base = head * D;                             // q heads, then k heads: both D wide, one after the other
-  for (int j = threadIdx.x; j < DP - pairs; j += blockDim.x) {
-    float a, bq = 0.f;
-    int d0, d1 = -1;
+  const int j = threadIdx.x;
+  float x0 = 0.f, x1 = 0.f;
+  int d0 = -1, d1 = -1;
+  if (j < DP - pairs) {
     if (j < pairs) {
       d0 = j;
       d1 = j + pairs;
-      const float x0 = value(base + d0), x1 = value(base + d1);
-      const float2 e = table[t * pairs + j];
-      const float cs = e.x * magnitude, sn = e.y * magnitude;
-      a = x0 * cs - x1 * sn;
-      bq = x1 * cs + x0 * sn;
+      x0 = value(base + d0);
+      x1 = value(base + d1);
     } else {
       d0 = j + pairs;
-      a = d0 < D ? value(base + d0) : 0.f;
+      if (d0 < D) x0 = value(base + d0);
     }
-    if (head < H) {
-      Q* q = q_out + (t * H + head) * DP;
-      const float qt = query_temperature(positions, t, temp_coef, temp_every);
-      q[d0] = from_float<Q>(a * qt);
-      if (d1 >= 0) q[d1] = from_float<Q>(bq * qt);
-    } else if (write && d0 < D) {
-      C* k = k_cache + ((page * G + (head - H)) * block_size + offset) * DP;
-      k[d0] = from_float<C>(to_float(from_float<Q>(a)));
-      if (d1 >= 0) k[d1] = from_float<C>(to_float(from_float<Q>(bq)));
-    }
+  }
+  const float* norm_weight = head < H ? q_norm : k_norm;
+  if (norm_weight != nullptr) {
+    // the norm over the head's D values, in float32, in front of the rotation
+    __shared__ float scratch[16];
+    const float r = 1.f / sqrtf(block_sum(x0 * x0 + x1 * x1, scratch) / D + norm_eps);
+    if (d0 >= 0 && d0 < D) x0 = x0 * r * norm_weight[d0];
+    if (d1 >= 0) x1 = x1 * r * norm_weight[d1];
+  }
+  if (d0 < 0) return;
+  float a = x0, bq = 0.f;
+  if (d1 >= 0) {
+    const float2 e = table[t * pairs + j];
+    const float cs = e.x * magnitude, sn = e.y * magnitude;
+    a = x0 * cs - x1 * sn;
+    bq = x1 * cs + x0 * sn;
+  }
+  if (head < H) {
+    Q* q = q_out + (t * H + head) * DP;
+    const float qt = query_temperature(positions, t, temp_coef, temp_every);
+    q[d0] = from_float<Q>(a * qt);
+    if (d1 >= 0) q[d1] = from_float<Q>(bq * qt);
+  } else if (write && d0 < D) {
+    C* k = k_cache + ((page * G + (head - H)) * block_size + offset) * DP;
+    k[d0] = from_float<C>(to_float(from_float<Q>(a)));
+    if (d1 >= 0) k[d1] = from_float<C>(to_float(from_float<Q>(bq)));
   }
 }
 
@@ -1073,9 +1089,13 @@ extern "C" int distie_conv_rope_kv_write(const void* product, int dtype, int64_t
                                          void* q_out, void* k_cache, void* v_cache, int cache_dtype, const int32_t* slots,
                                          const int32_t* cu_q, const int32_t* token_request, const int32_t* state_slots,
                                          int T, int H, int G, int D, int E, int DP, int block_size, int has_kv, int write,
-                                         const int32_t* positions, float temp_coef, int temp_every, hipStream_t stream) {
+                                         const int32_t* positions, float temp_coef, int temp_every, const float* q_norm,
+                                         const float* k_norm, float norm_eps, hipStream_t stream) {
   // temp_every >= 1: q of the token at position p times 1 + temp_coef * ln(floor((p + 1) / temp_every) + 1)
+  // q_norm / k_norm (float32 [D], null: none): every q / k head goes through x / sqrt(mean(x^2) + norm_eps) * weight
+  // over its D values, behind the convolution and in front of the rotation
   if (T <= 0) return 0;
+  if ((q_norm != nullptr || k_norm != nullptr) && !(norm_eps >= 0.f)) return DISTIE_BAD_ARGUMENT;
   if (temp_every >= 1 && positions == nullptr) return DISTIE_BAD_ARGUMENT;
   if (H < 1 || G < 1 || D < 1 || E < 1 || DP < D || DP < E || block_size < 1 || pairs < 0 || 2 * pairs > D ||
       taps < 0 || taps > MAX_TAPS)
@@ -1083,7 +1103,8 @@ extern "C" int distie_conv_rope_kv_write(const void* product, int dtype, int64_t
   if ((pairs > 0 && table == nullptr) || (taps > 1 && state == nullptr) || (taps >= 1 && weight == nullptr))
     return DISTIE_BAD_ARGUMENT;
   if (has_kv && write && (k_cache == nullptr || v_cache == nullptr || slots == nullptr)) return DISTIE_BAD_ARGUMENT;
-  if (dtype == DISTIE_BF16 && (weight == nullptr || w_dtype == DISTIE_BF16) && (!write || cache_dtype == DISTIE_BF16) &&
+  if (q_norm == nullptr && k_norm == nullptr &&
+      dtype == DISTIE_BF16 && (weight == nullptr || w_dtype == DISTIE_BF16) && (!write || cache_dtype == DISTIE_BF16) &&
       T >= 32 && D % 8 == 0 && E % 8 == 0 && DP % 8 == 0 && pairs % 8 == 0 && ld % 8 == 0 &&
       reinterpret_cast<uintptr_t>(product) % 16 == 0 && reinterpret_cast<uintptr_t>(q_out) % 16 == 0 && reinterpret_cast<uintptr_t>(k_cache) % 16 == 0 && reinterpret_cast<uintptr_t>(v_cache) % 16 == 0 && reinterpret_cast<uintptr_t>(state) % 16 == 0 && reinterpret_cast<uintptr_t>(table) % 16 == 0) {
     const int items = (has_kv ? H + G : H) * ((DP - pairs) / 8);
@@ -1104,7 +1125,8 @@ extern "C" int distie_conv_rope_kv_write(const void* product, int dtype, int64_t
       conv_rope_kv_write_kernel<X, W, X, C><<<grid, threads, 0, stream>>>(
           static_cast<const X*>(product), ld, static_cast<const W*>(weight), taps, state, static_cast<const float2*>(table),
           pairs, magnitude, static_cast<X*>(q_out), static_cast<C*>(k_cache), static_cast<C*>(v_cache), slots, cu_q,
-          token_request, state_slots, H, G, D, E, DP, block_size, has_kv, write, positions, temp_coef, temp_every))));
+          token_request, state_slots, H, G, D, E, DP, block_size, has_kv, write, positions, temp_coef, temp_every,
+          q_norm, k_norm, norm_eps))));
   return launch_status();
 }
 

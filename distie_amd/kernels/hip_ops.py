@@ -308,7 +308,7 @@ class HipOps(Ops):
         o.distie_causal_conv.argtypes = [_P, _I, _L, _P, _I, _I, _P, _P, _I, _L, _I, _P, _P, _P, _P, _I, _I, _P]
         o.distie_conv_state.argtypes = [_P, _I, _L, _I, _P, _P, _P, _I, _I, _I, _P]
         o.distie_conv_rope_kv_write.argtypes = [_P, _I, _L, _P, _I, _I, _P, _P, _I, _F, _P, _P, _P, _I, _P, _P, _P, _P,
-                                                _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _F, _I, _P]
+                                                _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _F, _I, _P, _P, _F, _P]
         o.distie_sigmoid_gate.argtypes = [_P, _I, _I, _I, _P, _I, _L, _P, _I, _I, _I, _P]
         o.distie_rmsnorm_gate.argtypes = [_P, _P, _I, _F, _P, _I, _L, _P, _I, _I, _I, _I, _I, _P]
         o.distie_norm_chain.argtypes = [_P, _I, _I, _P, _P, _I, _I, _P, _F, _F, _P, _F, _P, _P, _F, _P, _I, _P, _I, _I, _P]
@@ -317,7 +317,9 @@ class HipOps(Ops):
         o.distie_lru_gates.argtypes = [_P, _I, _L, _P, _P, _P, _P, _I, _P, _F, _P, _P, _I, _I, _I, _P]
         o.distie_lru_scan.argtypes = [_P, _P, _P, _P, _I, _L, _I, _P, _I, _P, _P, _I, _I, _P]
         o.distie_lru_scan_chunked.argtypes = [_P, _P, _P, _P, _P, _P, _P, _I, _L, _I, _P, _I, _P, _P, _P, _I, _I, _I, _P]
-        o.distie_route_topk.argtypes = [_P, _I, _P, _I, _P, _P, _P, _I, _I, _I, _I, _P]
+        o.distie_route_topk.argtypes = [_P, _I, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _P]
+        o.distie_route_glu.argtypes = [_P, _I, _L, _I, _P, _P, _I, _I, _I, _I, _F, _F, _F, _I, _P, _I, _P]
+        o.distie_softcap_f32.argtypes = [_P, _L, _F, _P]
         o.distie_route_scale.argtypes = [_P, _I, _L, _P, _P, _I, _I, _I, _I, _P]
         o.distie_scale_f32.argtypes = [_P, _L, _F, _P]
         o.distie_activation.argtypes = [_P, _I, _I, _P, _I, _L, _I, _P]
@@ -355,12 +357,12 @@ class HipOps(Ops):
                 raise KernelError(f"attention kernels take even head sizes up to 256, not {head_dim}")
             lib = ctypes.CDLL(str(build.ensure(f"attn_d{head_dim}")))
             lib.distie_attention_generic.argtypes = [_P, _I, _L, _P, _P, _I, _P, _P, _P, _I, _P, _P,
-                                                     _I, _I, _I, _I, _F, _I, _P, _F, _P]
+                                                     _I, _I, _I, _I, _F, _I, _P, _F, _P, _P]
             lib.distie_attention_prefill_bf16.argtypes = [_P, _L, _P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I,
-                                                          _F, _I, _I, _P, _P, _P, _I, _P]
+                                                          _F, _I, _I, _P, _P, _P, _I, _P, _P]
             lib.distie_attention_prefill_f32.argtypes = lib.distie_attention_prefill_bf16.argtypes
             lib.distie_attention_decode_bf16.argtypes = [_P, _L, _P, _P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I,
-                                                         _I, _F, _I, _I, _I, _I, _P, _P]
+                                                         _I, _F, _I, _I, _I, _I, _P, _P, _P]
             lib.distie_attention_decode_run_len.argtypes = [_P, _I, _I, _I, _P, _P]
             if lib.distie_attention_head_dim() != head_dim:
                 raise KernelError("attention library was built for another head size")
@@ -894,8 +896,9 @@ class HipOps(Ops):
 
     def paged_attention(self, qkv, meta: BatchMeta, group, k_cache, v_cache, num_heads, num_kv_heads, head_dim,
                         scale, window, extras=None):
-        """The matrix-core kernels and the tiled float32 kernel compute plain attention; a step with
-        `extras` goes to the wave-per-token kernel, which takes slopes and a cap (any types and sizes)."""
+        """The matrix-core kernels and the tiled float32 kernel compute attention with plain scores (a sink in the
+        denominator they take); a step whose `extras` bend the scores goes to the wave-per-token kernel, which takes
+        slopes and a cap as well (any types and sizes)."""
         if not scale > 0:
             raise KernelError(f"paged_attention: the scale of the scores must be positive, not {scale}")
         qkv = self.dense(qkv)
@@ -910,12 +913,15 @@ class HipOps(Ops):
             raise KernelError("paged_attention: tensors do not match the batch")
         rows_ptr = rows.data_ptr() if rows is not None else None
         out = torch.empty((T, num_heads * head_dim), dtype=qkv.dtype, device=self.device)
-        plain = extras is None or extras.plain
+        plain = extras is None or not extras.bends_scores
         slopes, cap = (None, 0.0) if plain else (extras.head_slopes, float(extras.score_cap or 0.0))
-        if slopes is not None:
-            self._own(slopes)
-            if slopes.dtype != torch.float32 or tuple(slopes.shape) != (num_heads,):
-                raise KernelError("paged_attention: head_slopes must be float32 [num_heads]")
+        sinks = extras.sinks if extras is not None else None
+        for name, vector in (("head_slopes", slopes), ("sinks", sinks)):
+            if vector is not None:
+                self._own(vector)
+                if vector.dtype != torch.float32 or tuple(vector.shape) != (num_heads,):
+                    raise KernelError(f"paged_attention: {name} must be float32 [num_heads]")
+        sinks_ptr = sinks.data_ptr() if sinks is not None else None
         bf16 = qkv.dtype == torch.bfloat16 and k_cache.dtype == torch.bfloat16
         if plain and bf16 and meta.block_size % 16 == 0 and head_dim % 16 == 0:
             # how the step is launched, and its buffers for partial results, are the same for every layer
@@ -934,7 +940,7 @@ class HipOps(Ops):
                     plan["decode_o"].data_ptr(), plan["decode_ml"].data_ptr(), meta.num_requests, num_heads,
                     num_kv_heads, meta.block_size, float(scale), int(window or 0), plan["split_len"],
                     plan["max_splits"], 1 if meta.all_decode else 0,
-                    plan["run_len"].data_ptr() if plan["run_len"] is not None else None, self._stream()),
+                    plan["run_len"].data_ptr() if plan["run_len"] is not None else None, sinks_ptr, self._stream()),
                     "attention_decode_bf16")
             if plan["prefill"]:
                 parts = plan["parts"]
@@ -944,7 +950,7 @@ class HipOps(Ops):
                     num_heads, num_kv_heads, meta.block_size, float(scale), int(window or 0),
                     2 if plan["decode"] else 1, meta.token_request.data_ptr(),
                     plan["prefill_o"].data_ptr() if parts > 1 else None,
-                    plan["prefill_ml"].data_ptr() if parts > 1 else None, parts, self._stream()),
+                    plan["prefill_ml"].data_ptr() if parts > 1 else None, parts, sinks_ptr, self._stream()),
                     "attention_prefill_bf16")
             return out
         f32 = qkv.dtype == torch.float32 and k_cache.dtype == torch.float32
@@ -962,13 +968,14 @@ class HipOps(Ops):
                 meta.cu_q.data_ptr(), table.data_ptr(), table.shape[1], rows_ptr, out.data_ptr(), T, meta.num_requests,
                 num_heads, num_kv_heads, meta.block_size, float(scale), int(window or 0), 1,
                 meta.token_request.data_ptr(), plan["prefill_o"].data_ptr() if parts > 1 else None,
-                plan["prefill_ml"].data_ptr() if parts > 1 else None, parts, self._stream()), "attention_prefill_f32")
+                plan["prefill_ml"].data_ptr() if parts > 1 else None, parts, sinks_ptr, self._stream()),
+                "attention_prefill_f32")
             return out
         _check(lib.distie_attention_generic(
             qkv.data_ptr(), _code(qkv), qkv.shape[1], k_cache.data_ptr(), v_cache.data_ptr(), _code(k_cache),
             meta.positions.data_ptr(), meta.token_request.data_ptr(), table.data_ptr(), table.shape[1], rows_ptr,
             out.data_ptr(), T, num_heads, num_kv_heads, meta.block_size, float(scale), int(window or 0),
-            slopes.data_ptr() if slopes is not None else None, cap, self._stream()), "attention_generic")
+            slopes.data_ptr() if slopes is not None else None, cap, sinks_ptr, self._stream()), "attention_generic")
         return out
 
     def _attention_plan(self, lib, meta: BatchMeta, T, num_heads, num_kv_heads, head_dim, window) -> dict:
@@ -1138,8 +1145,18 @@ class HipOps(Ops):
                               f"[slots, {taps - 1}, {channels}]")
 
     def conv_rope_kv_write(self, product, conv_weight, state, meta, group, k_cache, v_cache, inv_freq, magnitude,
-                           num_heads, num_kv_heads, dim, value_dim, padded_dim, has_kv, write, q_temp=None):
+                           num_heads, num_kv_heads, dim, value_dim, padded_dim, has_kv, write, q_temp=None, qk_norm=None):
         product = self.dense(product)
+        q_norm = k_norm = None
+        norm_eps = 0.0
+        if qk_norm is not None:
+            q_norm, k_norm, norm_eps = qk_norm
+            self._own(q_norm, k_norm)
+            for weight in (q_norm, k_norm):
+                if weight is not None and (weight.dtype != torch.float32 or tuple(weight.shape) != (dim,)):
+                    raise KernelError("conv_rope_kv_write: the norms' weights of q and k are float32 [dim]")
+            if q_norm is None or (has_kv and k_norm is None):
+                raise KernelError("conv_rope_kv_write: a norm on the heads needs a weight for q, and for k where there are keys")
         self._own(product, conv_weight, state, k_cache, v_cache, inv_freq)
         T, W = product.shape
         channels = num_heads * dim + (num_kv_heads * (dim + value_dim) if has_kv else 0)
@@ -1165,7 +1182,8 @@ class HipOps(Ops):
             meta.groups[group].slots.data_ptr() if write else None, meta.cu_q.data_ptr(), meta.token_request.data_ptr(),
             meta.state_slots.data_ptr(), T, num_heads, num_kv_heads, dim, value_dim, padded_dim, meta.block_size,
             1 if has_kv else 0, 1 if write else 0, meta.positions.data_ptr(), float(q_temp[0]) if q_temp else 0.0,
-            int(q_temp[1]) if q_temp else 0, self._stream()), "conv_rope_kv_write")
+            int(q_temp[1]) if q_temp else 0, ptr(q_norm), ptr(k_norm) if has_kv else None, float(norm_eps),
+            self._stream()), "conv_rope_kv_write")
         if taps > 1:
             if not meta.all_decode:
                 # (requests that bring one row had their state moved on by the kernel above)
@@ -1290,7 +1308,8 @@ class HipOps(Ops):
         out = y = None
         if residual is None:
             y = torch.empty((T, C), dtype=torch.float32, device=self.device)
-        elif pre is not None:
+        elif out_dtype is not None:
+            # with a norm in front of the next sub-layer (`pre`), or the new residual as it is, in `out_dtype`
             out = torch.empty((T, C), dtype=out_dtype, device=self.device)
         (t0, s0), (t1, s1) = held[0], (held[1] if len(held) > 1 else (None, 1))
         ptr = lambda t: t.data_ptr() if t is not None else None
@@ -1328,6 +1347,26 @@ class HipOps(Ops):
         if isinstance(delta, NormedSum):
             return self._norm_chain(delta.terms, delta.weights, delta.eps, delta.scale, post, residual, pre, out_dtype)
         return self._norm_chain([delta], None, 0.0, 1.0, post, residual, pre, out_dtype)
+
+    def read_residual(self, residual, out_dtype):
+        self._own(residual)
+        if residual.dtype != torch.float32 or residual.dim() != 2:
+            raise KernelError("read_residual reads the float32 residual stream")
+        if out_dtype == torch.float32:
+            return residual
+        out = torch.empty(residual.shape, dtype=out_dtype, device=self.device)
+        _check(self._ops.distie_sum_slices(residual.data_ptr(), 1, out.numel(), out.data_ptr(), _CODES[out_dtype],
+                                           self._stream()), "sum_slices")
+        return out
+
+    def add_normed_read(self, residual, delta, post_weight, post_eps, out_dtype):
+        if out_dtype == torch.float32:
+            self.add_normed(residual, delta, post_weight, post_eps)
+            return residual
+        post = (self._f32(post_weight), post_eps)
+        if isinstance(delta, NormedSum):
+            return self._norm_chain(delta.terms, delta.weights, delta.eps, delta.scale, post, residual, None, out_dtype)
+        return self._norm_chain([delta], None, 0.0, 1.0, post, residual, None, out_dtype)
 
     def gated_decay_scan(self, product, decay_logits, state, meta, num_heads, dim, value_dim, q_scale, tau, decay_low=None):
         product = self.dense(product)
@@ -1436,7 +1475,9 @@ class HipOps(Ops):
         _mark_written(state)
         return out
 
-    def route_topk(self, x, weight, bias, top):
+    def route_topk(self, x, weight, bias, top, scoring="softmax"):
+        if scoring not in ("softmax", "sigmoid"):
+            raise KernelError(f"route_topk: no scoring named {scoring!r}")
         x = self.dense(x)
         self._own(x, weight, bias)
         T, C = x.shape
@@ -1447,8 +1488,37 @@ class HipOps(Ops):
         gates = torch.empty((T, top), dtype=torch.float32, device=self.device)
         _check(self._ops.distie_route_topk(x.data_ptr(), _code(x), weight.data_ptr(), _code(weight),
                                            bias.data_ptr() if bias is not None else None, experts.data_ptr(),
-                                           gates.data_ptr(), T, C, E, int(top), self._stream()), "route_topk")
+                                           gates.data_ptr(), T, C, E, int(top), 1 if scoring == "sigmoid" else 0,
+                                           self._stream()), "route_topk")
         return experts, gates
+
+    def route_glu(self, gate_up, experts, gates, num_experts, width, limit, slope, up_shift, on_input):
+        if isinstance(gate_up, (PendingNorm, PendingProduct)):
+            gate_up = self.dense(gate_up)
+        slices, source, dtype = 1, gate_up, gate_up.dtype
+        if isinstance(gate_up, PartialSums):
+            slices, source = gate_up.slices, gate_up.data
+        self._own(source, experts, gates)
+        T, top = experts.shape
+        if experts.dtype != torch.int32 or gates.dtype != torch.float32 or gates.shape != experts.shape or \
+                gate_up.shape[0] != T or gate_up.shape[1] != 2 * num_experts * width:
+            raise KernelError("route_glu: experts int32 and gates float32 [T, top], gate_up [T, 2 * experts * width]")
+        if limit is not None and not limit > 0:
+            raise KernelError("route_glu: the limit must be positive")
+        out = torch.empty((T, num_experts * width), dtype=dtype, device=self.device)
+        _check(self._ops.distie_route_glu(source.data_ptr(), _code(source), gate_up.shape[1], slices, experts.data_ptr(),
+                                          gates.data_ptr(), T, top, num_experts, width, float(limit or 0.0), float(slope),
+                                          float(up_shift), 1 if on_input else 0, out.data_ptr(), _code(out),
+                                          self._stream()), "route_glu")
+        return out
+
+    def softcap(self, x, cap):
+        self._own(x)
+        if x.dtype != torch.float32:
+            raise KernelError("softcap works on float32 values")
+        _check(self._ops.distie_softcap_f32(x.data_ptr(), x.numel(), float(cap), self._stream()), "softcap_f32")
+        _mark_written(x)
+        return x
 
     def route_scale(self, hidden, experts, gates, num_experts, width):
         hidden = self.dense(hidden)

@@ -68,10 +68,13 @@ class ScoreExtras:
 
     score(i, j) = q_i . k_j * scale; with `score_cap` c: c * tanh(score / c); with `head_slopes` s:
     + s[h] * (j - i), a bias by the distance to the key with a slope of the head's own (a position
-    encoding that needs no rotation)."""
+    encoding that needs no rotation). With `sinks` z: the softmax's denominator holds exp(z[h]) beside the
+    visible keys' terms, weight(i, j) = exp(score(i, j)) / (exp(z[h]) + sum_j' exp(score(i, j'))); the sink is
+    not scaled, has no value and counts once for every query, whatever its window."""
 
     head_slopes: Optional[torch.Tensor] = None      # float32 [H] on the device
     score_cap: Optional[float] = None               # > 0
+    sinks: Optional[torch.Tensor] = None            # float32 [H] on the device
 
     def __post_init__(self):
         if self.score_cap is not None and not self.score_cap > 0:
@@ -79,7 +82,12 @@ class ScoreExtras:
 
     @property
     def plain(self) -> bool:
-        return self.head_slopes is None and self.score_cap is None
+        return self.head_slopes is None and self.score_cap is None and self.sinks is None
+
+    @property
+    def bends_scores(self) -> bool:
+        """Something changes the scores themselves (a sink does not: it only joins the denominator)."""
+        return self.head_slopes is not None or self.score_cap is not None
 
 
 class Ops(abc.ABC):
@@ -218,7 +226,7 @@ class Ops(abc.ABC):
                            k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
                            inv_freq: Optional[torch.Tensor], magnitude: float, num_heads: int, num_kv_heads: int,
                            dim: int, value_dim: int, padded_dim: int, has_kv: bool, write: bool,
-                           q_temp=None) -> torch.Tensor:
+                           q_temp=None, qk_norm=None) -> torch.Tensor:
         """Behind attention's stacked projection. The first columns of `product` (act [T, W]) are q (num_heads x
         dim) and, if `has_kv`, k (num_kv_heads x dim) and v (num_kv_heads x value_dim); further columns are left
         alone. Each of these channels goes through `causal_conv` (no residual; `conv_weight` [channels, taps],
@@ -228,7 +236,10 @@ class Ops(abc.ABC):
         v_cache [pages, KH, padded_dim, P]. Returns q as act [T, num_heads * padded_dim], zeros beyond `dim`:
         what `paged_attention` reads with a head size of `padded_dim`.
         `q_temp` = (coef, every): a query temperature by position, q of the token at position p is multiplied by
-        1 + coef * ln(floor((p + 1) / every) + 1), computed in float32 (None: none)."""
+        1 + coef * ln(floor((p + 1) / every) + 1), computed in float32 (None: none).
+        `qk_norm` = (q_weight float32 [dim], k_weight float32 [dim] or None without keys, eps): behind the convolution
+        and in front of the rotation every q and k head becomes x / sqrt(mean(x^2) + eps) * weight over its `dim`
+        values, in float32 (None: none)."""
         raise NotImplementedError(f"{type(self).__name__} has no convolution over time")
 
     def sigmoid_gate(self, x: torch.Tensor, num_heads: int, head_stride: int, width: int,
@@ -267,6 +278,17 @@ class Ops(abc.ABC):
         """residual (float32 [T, C], in place) += rmsnorm(delta) * weight: a sub-layer's result with a norm behind
         it. `delta`: act [T, C], what `linear` returned, or what `normed_sum` returned."""
         raise NotImplementedError(f"{type(self).__name__} has no norm behind a sub-layer")
+
+    def read_residual(self, residual: torch.Tensor, out_dtype) -> torch.Tensor:
+        """The residual (float32 [T, C]) as a sub-layer without a norm in front reads it: rounded to `out_dtype`,
+        or the tensor itself where that is float32."""
+        return residual if out_dtype == residual.dtype else residual.to(out_dtype)
+
+    def add_normed_read(self, residual: torch.Tensor, delta, post_weight: torch.Tensor, post_eps: float,
+                        out_dtype) -> torch.Tensor:
+        """`add_normed`, then `read_residual`; an implementation may fuse the two."""
+        self.add_normed(residual, delta, post_weight, post_eps)
+        return self.read_residual(residual, out_dtype)
 
     def add_normed_rmsnorm(self, residual: torch.Tensor, delta, post_weight: torch.Tensor, post_eps: float,
                            weight: torch.Tensor, eps: float, out_dtype) -> torch.Tensor:
@@ -309,11 +331,26 @@ class Ops(abc.ABC):
         one of `activation`'s names or None for mul itself; `mul` None: h)."""
         raise NotImplementedError(f"{type(self).__name__} has no gated linear recurrent unit")
 
-    def route_topk(self, x, weight: torch.Tensor, bias: Optional[torch.Tensor], top: int):
+    def route_topk(self, x, weight: torch.Tensor, bias: Optional[torch.Tensor], top: int, scoring: str = "softmax"):
         """The router of a mixture of experts: z = weight x + bias in float32 (x act [T, C], weight [E, C], bias
-        float32 [E]); for every row the `top` largest z (the lower index among equals) and softmax over those alone
+        float32 [E] or None); for every row the `top` largest z (the lower index among equals) and, as weights,
+        softmax over those alone (`scoring` "softmax") or sigmoid(z) of each, not renormalised ("sigmoid")
         -> (experts int32 [T, top], their weights float32 [T, top]), largest first."""
         raise NotImplementedError(f"{type(self).__name__} has no router")
+
+    def route_glu(self, gate_up, experts: torch.Tensor, gates: torch.Tensor, num_experts: int, width: int,
+                  limit: Optional[float], slope: float, up_shift: float, on_input: bool) -> torch.Tensor:
+        """The hidden values of routed gated experts from the stacked product. `gate_up` act [T, 2 * num_experts *
+        width] (or what `linear` returned): every expert's gate columns, expert after expert, then every expert's up
+        columns. For expert e of a row with weight w (zero result if the row did not choose e):
+        g, u = gate and up columns, times w if `on_input`; with `limit`: g <- min(g, limit), u <- clamp(u, -limit,
+        limit); hidden = g * sigmoid(slope * g) * (u + up_shift), times w unless `on_input`
+        -> act [T, num_experts * width], in float32 behind the product's rounding."""
+        raise NotImplementedError(f"{type(self).__name__} has no routed feed-forward")
+
+    def softcap(self, x: torch.Tensor, cap: float) -> torch.Tensor:
+        """float32 [R, N] (in place) -> cap * tanh(x / cap)."""
+        raise NotImplementedError(f"{type(self).__name__} has no cap on values")
 
     def route_scale(self, hidden: torch.Tensor, experts: torch.Tensor, gates: torch.Tensor, num_experts: int,
                     width: int) -> torch.Tensor:

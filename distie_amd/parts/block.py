@@ -208,6 +208,55 @@ class SandwichResidual(Block):
         stream.lanes["pending"] = (y, self.feed_forward_post_norm)
 
 
+class BranchNormResidual(Block):
+    """A norm on each sub-layer's result only, inside the residual branch; the sub-layers read the residual itself:
+
+        x <- x + mixer_post_norm(mixer(x));   x <- x + feed_forward_post_norm(feed_forward(x))
+
+    Both are RMS norms. A layer may have no feed-forward. The residual is float32; a sub-layer reads it rounded to
+    the activations' precision (itself in a float32 engine). A sub-layer's result stays pending with its norm, and
+    the read for the next sub-layer adds it (`Ops.add_normed_read`: one kernel between two sub-layers); the model's
+    last norm finds the plain sum through `ResidualStream.close`."""
+
+    CHILDREN = {"mixer": "mixer", "mixer_post_norm": "norm", "feed_forward": "feed_forward",
+                "feed_forward_post_norm": "norm"}
+    OPTIONAL = ("feed_forward", "feed_forward_post_norm")
+
+    def __init__(self, spec, parts) -> None:
+        super().__init__(spec, parts)
+        if (self.feed_forward is None) != (self.feed_forward_post_norm is None):
+            raise ValueError("a feed-forward and its norm come together")
+        for norm in (self.mixer_post_norm, self.feed_forward_post_norm):
+            if norm is not None and getattr(norm, "fused_kind", None) != "rms":
+                raise ValueError("the branch-norm arrangement takes RMS norms")
+
+    _settle = staticmethod(SandwichResidual._settle)
+
+    @staticmethod
+    def _read(ops, stream: ResidualStream, act_dtype):
+        """Add what is pending, through its norm, and hand out the residual in the activations' precision."""
+        if stream.pending is not None:
+            raise ValueError("the branch-norm arrangement starts from a residual with nothing pending on it")
+        pending = stream.lanes.get("pending") if stream.lanes else None
+        if pending is None:
+            return ops.read_residual(stream.hidden, act_dtype)
+        delta, post = pending
+        stream.lanes["pending"] = None
+        return ops.add_normed_read(stream.hidden, delta, post.weight, post.eps, act_dtype)
+
+    def forward(self, ops, stream: ResidualStream, ctx: StepContext, cache, writes_cache: bool) -> None:
+        h = self._read(ops, stream, ctx.act_dtype)
+        y = self.mixer.forward(ops, h, ctx, cache["mixer"], writes_cache)
+        stream.lanes = {"pending": (y, self.mixer_post_norm)}
+        stream.settle = self._settle
+        if self.feed_forward is None:
+            return
+        h = self._read(ops, stream, ctx.act_dtype)
+        y = self.feed_forward.forward(ops, h, ctx)
+        stream.lanes["pending"] = (y, self.feed_forward_post_norm)
+
+
 register_part("block", "prenorm_residual", PreNormResidual)
+register_part("block", "branch_norm_residual", BranchNormResidual)
 register_part("block", "sandwich_residual", SandwichResidual)
 register_part("block", "hyper_connections", HyperConnections)

@@ -10,6 +10,11 @@
 * biases on q, k and v (`bias`: tensors `<q|k|v>.b`, added in the projection);
 * a query temperature by position (`q_temp` = {coef, every}): q at position p is multiplied by
   1 + coef * ln(floor((p + 1) / every) + 1), in float32, so that later queries weigh their keys more sharply;
+* a norm on every head of q and k (`qk_norm` = {eps, offset}): RMS norm over the head's `head_dim` values with the
+  weights `q.norm` and `k.norm` [head_dim] (each shared by all heads; `offset` is added to the stored weight),
+  behind the convolution and before the rotation, in float32;
+* a sink in the softmax (`sink`): a learned number per query head (`sink` [heads]) whose exponential is one more term
+  of the denominator; it has no key and no value, is not scaled, and counts once whatever the window;
 * keys and values borrowed from an earlier layer (`kv_from`): such a layer has no k or v tensors; it reads the other
   layer's cache (keys as they lie there, convolved and rotated; values convolved) with queries, window and everything
   else of its own. The lending layer must keep its pages for as long as a borrower looks back (`keep`).
@@ -27,6 +32,7 @@ import bisect
 import torch
 
 from ..config.model_config import PartSpec
+from ..kernels.interface import ScoreExtras
 from .attention import PagedKV, context_classes
 from .base import Borrowed, CacheNeeds, FixedState, Mixer, ParamSpec, TensorDecl, build_part, register_part
 
@@ -63,6 +69,10 @@ class ConvGatedAttention(Mixer):
             raise ValueError("q_temp.every must be >= 1")
         if self.num_heads % self.num_kv_heads:
             raise ValueError("num_heads must be a multiple of num_kv_heads")
+        norm = p.get("qk_norm")
+        self.qk_norm = (float(norm["eps"]), float(norm.get("offset") or 0.0)) if norm else None
+        self.sink = bool(p.get("sink", False))
+        self.q_norm_weight = self.k_norm_weight = self.extras = None
         self.position = build_part("position", p.get("position") or PartSpec("none"))
         self.padded_dim = padded_head_dim(self.head_dim, self.value_dim)
         self.has_kv = self.kv_from is None
@@ -92,6 +102,13 @@ class ConvGatedAttention(Mixer):
         if self.conv_taps:
             for name, rows in self._projections():
                 specs[name + ".conv"] = ParamSpec((rows, self.conv_taps))
+        if self.qk_norm is not None:
+            init = "zeros" if self.qk_norm[1] else "ones"
+            specs["q.norm"] = ParamSpec((self.head_dim,), init)
+            if self.has_kv:
+                specs["k.norm"] = ParamSpec((self.head_dim,), init)
+        if self.sink:
+            specs["sink"] = ParamSpec((self.num_heads,))
         if self.output_gate:
             specs["g"] = ParamSpec((self.gate_width, self.hidden_size))
         specs["o"] = ParamSpec((self.hidden_size, self.gate_width))
@@ -109,6 +126,12 @@ class ConvGatedAttention(Mixer):
         if self.conv_taps:
             self.conv_weight = torch.cat([tensors[name + ".conv"] for name, _ in self._projections()], dim=0).contiguous()
         self.out_weight = tensors["o"].contiguous()
+        if self.qk_norm is not None:
+            self.q_norm_weight = (tensors["q.norm"].float() + self.qk_norm[1]).contiguous()
+            if self.has_kv:
+                self.k_norm_weight = (tensors["k.norm"].float() + self.qk_norm[1]).contiguous()
+        if self.sink:
+            self.extras = ScoreExtras(sinks=tensors["sink"].float().contiguous())
         self.position.to_device(self.out_weight.device)
 
     def prepare(self, ops) -> None:
@@ -126,9 +149,10 @@ class ConvGatedAttention(Mixer):
         q = ops.conv_rope_kv_write(product, self.conv_weight, state, ctx.meta, cache.group, k_cache, v_cache,
                                    self.position.rotary(), self.position.rotary_magnitude(), self.num_heads,
                                    self.num_kv_heads, self.head_dim, self.value_dim, self.padded_dim, self.has_kv,
-                                   writes_cache and self.has_kv, self.q_temp)
+                                   writes_cache and self.has_kv, self.q_temp,
+                                   None if self.qk_norm is None else (self.q_norm_weight, self.k_norm_weight, self.qk_norm[0]))
         mixed = ops.paged_attention(q, ctx.meta, cache.group, k_cache, v_cache, self.num_heads, self.num_kv_heads,
-                                    self.padded_dim, self.scale, self.window)
+                                    self.padded_dim, self.scale, self.window, self.extras)
         if self.output_gate:
             gates = product[:, self.conv_channels:self.conv_channels + self.gate_width]
             mixed = ops.sigmoid_gate(mixed, self.num_heads, self.padded_dim, self.value_dim, gates)

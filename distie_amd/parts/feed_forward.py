@@ -79,6 +79,13 @@ class RoutedExperts(FeedForward):
     [F, C] and `e<e>.down` [C, F], no biases. `shared_size` > 0: one more expert of that size (`shared.*`) that every
     token uses with weight one.
 
+    Variants, each a parameter: `router_bias` False: no `router.b`. `scoring` "sigmoid": an expert's weight is
+    sigmoid(z) of its own logit, not renormalised over the chosen (the `top` largest scores are the `top` largest
+    logits). `weight_on` "input": the weight multiplies what the expert reads, expert(w x), instead of what it
+    returns. `activation` "clamped_glu": with g = min(gate x, limit) and u = clamp(up x, -limit, limit) the hidden
+    values are g * sigmoid(slope * g) * (u + up_shift). Since gate and up are linear, gate (w x) = w (gate x): the
+    weight is applied to the stacked product's columns, in float32, in front of the clamps.
+
     All experts' gate and up weights are stacked into one matrix (the shared expert's behind them), all down weights
     side by side into another: one product gives every expert's hidden values for every token, those of the experts a
     token did not choose are multiplied by zero and the chosen ones by their weight, and the second product adds
@@ -95,6 +102,22 @@ class RoutedExperts(FeedForward):
         self.shared_size = int(p.get("shared_size") or 0)
         if not 1 <= self.top <= self.num_experts:
             raise ValueError("a token uses between one and all of the experts")
+        self.has_router_bias = bool(p.get("router_bias", True))
+        self.scoring = str(p.get("scoring", "softmax"))
+        self.weight_on = str(p.get("weight_on", "output"))
+        self.activation = str(p.get("activation", "silu_glu"))
+        if self.scoring not in ("softmax", "sigmoid") or self.weight_on not in ("input", "output") or \
+                self.activation not in ("silu_glu", "clamped_glu"):
+            raise ValueError("routed experts: scoring is softmax or sigmoid, weight_on input or output, activation "
+                             "silu_glu or clamped_glu")
+        self.plain = self.activation == "silu_glu" and self.weight_on == "output"
+        if not self.plain and self.shared_size:
+            raise ValueError("routed experts: a shared expert goes with the plain gated activation only")
+        self.limit = float(p.get("limit") or 0.0)
+        self.slope = float(p.get("slope", 1.0))
+        self.up_shift = float(p.get("up_shift", 0.0))
+        if self.activation == "clamped_glu" and not self.limit > 0:
+            raise ValueError("routed experts: the clamped activation needs a positive limit")
         self.router_weight = self.router_bias = self.gate_up_weight = self.down_weight = None
 
     def _experts(self):
@@ -102,7 +125,9 @@ class RoutedExperts(FeedForward):
             ([("shared.", self.shared_size)] if self.shared_size else [])
 
     def param_specs(self):
-        specs = {"router": ParamSpec((self.num_experts, self.hidden_size)), "router.b": ParamSpec((self.num_experts,))}
+        specs = {"router": ParamSpec((self.num_experts, self.hidden_size))}
+        if self.has_router_bias:
+            specs["router.b"] = ParamSpec((self.num_experts,))
         for prefix, size in self._experts():
             specs[prefix + "gate"] = ParamSpec((size, self.hidden_size))
             specs[prefix + "up"] = ParamSpec((size, self.hidden_size))
@@ -111,7 +136,7 @@ class RoutedExperts(FeedForward):
 
     def load(self, tensors) -> None:
         self.router_weight = tensors["router"].contiguous()
-        self.router_bias = tensors["router.b"].float().contiguous()
+        self.router_bias = tensors["router.b"].float().contiguous() if self.has_router_bias else None
         names = [prefix for prefix, _ in self._experts()]
         stacked = [tensors[n + "gate"] for n in names] + [tensors[n + "up"] for n in names]
         dtype = torch.float32 if any(t.dtype == torch.float32 for t in stacked) else stacked[0].dtype
@@ -121,12 +146,17 @@ class RoutedExperts(FeedForward):
         self.down_weight = torch.cat([t.to(dtype) for t in down], dim=1).contiguous()
 
     def prepare(self, ops) -> None:
-        ops.prepare_linear(self.gate_up_weight, gated=True, role="gate_up")
+        ops.prepare_linear(self.gate_up_weight, gated=self.plain, role="gate_up")
         ops.prepare_linear(self.down_weight, role="down")
 
     def forward(self, ops, x, ctx):
         x = ops.dense(x)
-        experts, gates = ops.route_topk(x, self.router_weight, self.router_bias, self.top)
+        experts, gates = ops.route_topk(x, self.router_weight, self.router_bias, self.top, self.scoring)
+        if not self.plain:
+            hidden = ops.route_glu(ops.linear(x, self.gate_up_weight), experts, gates, self.num_experts,
+                                   self.expert_size, self.limit if self.activation == "clamped_glu" else None,
+                                   self.slope, self.up_shift, self.weight_on == "input")
+            return ops.linear(hidden, self.down_weight)
         hidden = ops.dense(ops.linear_silu_mul(x, self.gate_up_weight))
         hidden = ops.route_scale(hidden, experts, gates, self.num_experts, self.expert_size)
         return ops.linear(hidden, self.down_weight)

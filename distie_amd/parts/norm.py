@@ -10,6 +10,9 @@ from .base import Norm, ParamSpec, register_part
 
 
 class RMSNorm(Norm):
+    """`offset`: what is added to the stored weight (1 for designs whose files hold the weight minus one:
+    y = x / rms(x) * (1 + w)); the sum is made once at load, in float32, and is the weight from then on."""
+
     fused_kind = "rms"          # what `Ops.hyper_step` calls this norm when it computes it while reading the streams
 
     def __init__(self, spec) -> None:
@@ -17,13 +20,16 @@ class RMSNorm(Norm):
         self.size = int(spec.params["size"])
         self.eps = float(spec.params["eps"])
         self.weight_name = spec.params.get("weight_name", "weight")      # the tensor's name behind the prefix
+        self.offset = float(spec.params.get("offset") or 0.0)
         self.weight = None
 
     def param_specs(self):
-        return {self.weight_name: ParamSpec((self.size,), "ones")}
+        return {self.weight_name: ParamSpec((self.size,), "zeros" if self.offset else "ones")}
 
     def load(self, tensors) -> None:
         self.weight = tensors[self.weight_name].contiguous()
+        if self.offset:
+            self.weight = (self.weight.float() + self.offset).contiguous()
 
     def apply(self, ops, x, out_dtype):
         return ops.rmsnorm(x, self.weight, self.eps, out_dtype)

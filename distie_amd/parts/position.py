@@ -87,10 +87,52 @@ class ScaledRotaryPosition(PositionEncoding):
         return self.magnitude
 
 
+class BandedRotaryPosition(PositionEncoding):
+    """Rotation of the first `dims` dimensions of a head, with the frequencies scaled by bands of wavelength:
+    f_i = base^(-2i/dims), wavelength l_i = 2 pi / f_i. With `scaling` = {factor, low, high, original}: a frequency
+    whose wavelength is shorter than original / high stays; one whose wavelength is longer than original / low
+    becomes f_i / factor; between the two, with s = (original / l_i - low) / (high - low), it becomes
+    (1 - s) f_i / factor + s f_i. Computed in float64 and rounded once. Without `scaling`: plain rotation."""
+
+    def __init__(self, spec) -> None:
+        super().__init__(spec)
+        p = spec.params
+        self.dims = int(p["dims"])
+        self.base = float(p["base"])
+        if self.dims < 2 or self.dims % 2:
+            raise ValueError("rotary dimension must be even")
+        scaling = p.get("scaling")
+        freqs = []
+        for i in range(self.dims // 2):
+            f = self.base ** (-2.0 * i / self.dims)
+            if scaling:
+                factor, original = float(scaling["factor"]), float(scaling["original"])
+                low, high = float(scaling["low"]), float(scaling["high"])
+                length = 2 * math.pi / f
+                if length > original / low:
+                    f = f / factor
+                elif not length < original / high:
+                    s = (original / length - low) / (high - low)
+                    f = (1 - s) * f / factor + s * f
+            freqs.append(f)
+        self.inv_freq = torch.tensor(freqs, dtype=torch.float64).to(torch.float32)
+        self._key = (self.dims, self.base, repr(sorted(scaling.items())) if scaling else None)
+
+    def to_device(self, device) -> None:
+        key = ("banded",) + self._key + (str(device),)
+        if key not in _SHARED:
+            _SHARED[key] = self.inv_freq.to(device)
+        self.inv_freq = _SHARED[key]
+
+    def rotary(self):
+        return self.inv_freq
+
+
 class NoPosition(PositionEncoding):
     """For mixers whose order comes from elsewhere (a state, a learned table)."""
 
 
 register_part("position", "rope", RotaryPosition)
 register_part("position", "rope_scaled", ScaledRotaryPosition)
+register_part("position", "rope_banded", BandedRotaryPosition)
 register_part("position", "none", NoPosition)

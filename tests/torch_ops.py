@@ -89,7 +89,11 @@ class TorchOps(Ops):
                     s = extras.score_cap * torch.tanh(s / extras.score_cap)
                 if extras is not None and extras.head_slopes is not None:
                     s = s + extras.head_slopes.float()[:, None] * (keys - pos).float()[None, :]
-                out[t] = torch.einsum("hn,nhd->hd", torch.softmax(s, -1), v)
+                if extras is not None and extras.sinks is not None:
+                    w = torch.softmax(torch.cat([s, extras.sinks.float()[:, None]], -1), -1)[:, :-1]
+                else:
+                    w = torch.softmax(s, -1)
+                out[t] = torch.einsum("hn,nhd->hd", w, v)
         return out.view(T, num_heads * head_dim).to(qkv.dtype)
 
     # ---- residual streams, convolutions over time, decayed states, gates
@@ -141,7 +145,7 @@ class TorchOps(Ops):
         return (y if bias is None else y + bias.float()).to(x.dtype)
 
     def conv_rope_kv_write(self, product, conv_weight, state, meta, group, k_cache, v_cache, inv_freq, magnitude,
-                           num_heads, num_kv_heads, dim, value_dim, padded_dim, has_kv, write, q_temp=None):
+                           num_heads, num_kv_heads, dim, value_dim, padded_dim, has_kv, write, q_temp=None, qk_norm=None):
         T = product.shape[0]
         channels = num_heads * dim + (num_kv_heads * (dim + value_dim) if has_kv else 0)
         u = product[:, :channels]
@@ -157,14 +161,20 @@ class TorchOps(Ops):
             a, b = x[..., :pairs], x[..., pairs:2 * pairs]
             return torch.cat([a * cos - b * sin, b * cos + a * sin, x[..., 2 * pairs:]], -1)
 
+        def normed(x, weight):
+            if qk_norm is None:
+                return x
+            return x / torch.sqrt((x * x).mean(-1, keepdim=True) + qk_norm[2]) * weight.float()
+
         q = torch.zeros(T, num_heads, padded_dim, dtype=torch.float32, device=product.device)
-        q[..., :dim] = turned(u[:, :num_heads * dim].reshape(T, num_heads, dim))
+        q[..., :dim] = turned(normed(u[:, :num_heads * dim].reshape(T, num_heads, dim), qk_norm and qk_norm[0]))
         if q_temp is not None:
             coef, every = q_temp
             steps = torch.div(meta.positions.long() + 1, int(every), rounding_mode="floor")
             q = q * (1.0 + float(coef) * torch.log(steps.float() + 1.0))[:, None, None]
         if has_kv and write:
-            k = turned(u[:, num_heads * dim:(num_heads + num_kv_heads) * dim].reshape(T, num_kv_heads, dim))
+            k = turned(normed(u[:, num_heads * dim:(num_heads + num_kv_heads) * dim].reshape(T, num_kv_heads, dim),
+                              qk_norm and qk_norm[1]))
             v = u[:, (num_heads + num_kv_heads) * dim:].reshape(T, num_kv_heads, value_dim)
             P = k_cache.shape[2]
             slots = meta.groups[group].slots.long()
@@ -256,12 +266,35 @@ class TorchOps(Ops):
             out = out * (mul.float() if mul_act is None else self.activation(mul.float(), mul_act))
         return out.to(out_dtype)
 
-    def route_topk(self, x, weight, bias, top):
+    def route_topk(self, x, weight, bias, top, scoring="softmax"):
         z = x.float() @ weight.float().T
         if bias is not None:
             z = z + bias.float()
         order = torch.sort(z, dim=-1, descending=True, stable=True).indices[:, :top]
-        return order.to(torch.int32), torch.softmax(torch.gather(z, 1, order), -1)
+        chosen = torch.gather(z, 1, order)
+        return order.to(torch.int32), torch.sigmoid(chosen) if scoring == "sigmoid" else torch.softmax(chosen, -1)
+
+    def route_glu(self, gate_up, experts, gates, num_experts, width, limit, slope, up_shift, on_input):
+        T = gate_up.shape[0]
+        factor = torch.zeros(T, num_experts, dtype=torch.float32, device=gate_up.device)
+        factor.scatter_(1, experts.long(), gates.float())
+        chosen = torch.zeros(T, num_experts, dtype=torch.bool, device=gate_up.device)
+        chosen.scatter_(1, experts.long(), True)
+        g = gate_up[:, :num_experts * width].float().view(T, num_experts, width)
+        u = gate_up[:, num_experts * width:].float().view(T, num_experts, width)
+        if on_input:
+            g, u = g * factor[:, :, None], u * factor[:, :, None]
+        if limit is not None:
+            g, u = g.clamp(max=limit), u.clamp(-limit, limit)
+        hidden = g * torch.sigmoid(slope * g) * (u + up_shift)
+        if not on_input:
+            hidden = hidden * factor[:, :, None]
+        hidden = torch.where(chosen[:, :, None], hidden, torch.zeros_like(hidden))
+        return hidden.view(T, -1).to(gate_up.dtype)
+
+    def softcap(self, x, cap):
+        x.copy_(cap * torch.tanh(x / cap))
+        return x
 
     def route_scale(self, hidden, experts, gates, num_experts, width):
         T = hidden.shape[0]
