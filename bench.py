@@ -17,8 +17,8 @@ serves it), points at batch 1 and 32, and a cache that takes the card's memory u
 the time to the first token and the time per output token after it, defined as the reference's load
 generator defines them (benchmarks/load/stats.py:29-34, 67-86).
 
-`--design musutar|duparax [--size w1024|w2048|w4096]`: prefill and decode of that decoder beside a Qwen2 decoder of
-equal width, depth, heads and weights, at layer sizes of real models; one JSON line with both for every size.
+`--design musutar|duparax|sekazen [--size w1024|w2048|w4096]`: prefill and decode of that decoder beside a Qwen2
+decoder of equal width, depth, heads and weights, at layer sizes of real models; one JSON line with both for every size.
 
 Random weights N(0, 0.02), seeded uniform token ids.
 """
@@ -260,6 +260,24 @@ def duparax_config(size):
             "logit_scale": 0.5, "layers": layers}
 
 
+def sekazen_config(size):
+    """Pairs of windowed attention layers with head norms and sinks, the second of a pair on the first one's keys and
+    values; every layer's feed-forward is a mixture of eight clamped gated experts of a quarter of the dense size, two
+    a token, weighted by their own sigmoid scores on the input."""
+    z = DESIGN_SIZES[size]
+    rot = {"base": 150000.0, "dims": z["dim"] // 2, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}
+    layers = []
+    for i in range(z["layers"]):
+        mixer = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["dim"],
+                 "mask": {"size": z["window"]}, "rot": rot, "scale": z["dim"] ** -0.5}
+        if i % 2 == 1:
+            mixer["kv_from"] = i - 1
+        layers.append({"type": "attention", "mixer": mixer,
+                       "mlp": {"kind": "moe", "router": {"experts": 8, "top": 2}, "expert": {"ff": z["ff"] // 4, "limit": 7.0}}})
+    return {"architecture": "Sekazen", "vocab": DESIGN_VOCAB, "width": z["width"], "norm": {"eps": 1e-6},
+            "logit_softcap": 50.0, "layers": layers}
+
+
 def qwen2_of_weights(size, layer_weights):
     """The Qwen2 decoder with the same width, depth and heads and a feed-forward sized so that its layers hold as many
     weights as the other design's layers do on average."""
@@ -278,7 +296,7 @@ def design_pair(design, size):
     from distie_amd.config import config_from_dict
     from distie_amd.engine.model import Model
 
-    config = duparax_config(size)
+    config = sekazen_config(size) if design == "sekazen" else duparax_config(size)
     total = 0
     for name, spec in Model.declare(config_from_dict(config).model_spec()).items():
         if name.startswith("l"):
@@ -350,7 +368,7 @@ def main() -> int:
                         help="size the cache from free memory (the default for --shape 32b and --serve: 0.9)")
     parser.add_argument("--packed-weights", default=None, metavar="ROLES",
                         help="packed copies only for these products (qkv,attn_out,gate_up,down,head); 'none' for no copies")
-    parser.add_argument("--design", default=None, choices=["musutar", "duparax"],
+    parser.add_argument("--design", default=None, choices=["musutar", "duparax", "sekazen"],
                         help="instead of the workload above: this design beside a Qwen2 decoder of equal size, prefill and decode")
     parser.add_argument("--size", default=None, choices=sorted(DESIGN_SIZES), help="with --design: one size instead of all")
     args = parser.parse_args()

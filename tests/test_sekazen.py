@@ -105,7 +105,7 @@ ODD = su.make_config([
              scaled=su.scaling(factor=8.0, low=0.5, high=3.0, original=40), mlp=su.moe(experts=7, top=2, ff=10, limit=1.5)),
     su.layer(heads=5, kv_heads=1, dim=20, vdim=12, scale=0.35, window=3, dims=6, base=30.0,
              scaled=su.scaling(factor=8.0, low=0.5, high=3.0, original=40), kv_from=0, mlp=su.moe(experts=2, top=1, ff=6)),
-], vocab=50, width=40, cap=30.0)
+], vocab=50, width=40, cap=20.0)
 
 CONFIGS = {"mixed": MIXED, "plain": PLAIN, "odd": ODD}
 
