@@ -38,10 +38,18 @@ __device__ __forceinline__ float activate(float z, int kind) {   // the kinds of
 // they are read again where they are needed.
 constexpr int NORM_HELD_MAX = 8192;
 
-// V values at p as floats: V = 4 takes one 16-byte (float32) or 8-byte (bfloat16) load
+// V values at p as floats: V = 4 takes one 16-byte (float32) or 8-byte (bfloat16) load, V = 8 two or one of 16 bytes
 template <int V, typename T>
 __device__ __forceinline__ void load_values(const T* __restrict__ p, float out[V]) {
-  if constexpr (V == 4 && sizeof(T) == 4) {
+  if constexpr (V == 8 && sizeof(T) == 4) {
+    load_values<4>(p, out);
+    load_values<4>(p + 4, out + 4);
+  } else if constexpr (V == 8) {
+    const uint4 v = *reinterpret_cast<const uint4*>(p);
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int k = 0; k < 4; ++k) out[2 * k] = __uint_as_float(w[k] << 16), out[2 * k + 1] = __uint_as_float(w[k] & 0xffff0000u);
+  } else if constexpr (V == 4 && sizeof(T) == 4) {
     const float4 v = *reinterpret_cast<const float4*>(p);
     out[0] = v.x, out[1] = v.y, out[2] = v.z, out[3] = v.w;
   } else if constexpr (V == 4) {
@@ -56,13 +64,18 @@ __device__ __forceinline__ void load_values(const T* __restrict__ p, float out[V
 
 template <int V, typename T>
 __device__ __forceinline__ void store_values(T* __restrict__ p, const float v[V]) {
-  if constexpr (V == 4 && sizeof(T) == 4) {
+  const auto word = [](float lo, float hi) {
+    return static_cast<uint32_t>(__builtin_bit_cast(uint16_t, static_cast<bf16_t>(lo))) |
+           (static_cast<uint32_t>(__builtin_bit_cast(uint16_t, static_cast<bf16_t>(hi))) << 16);
+  };
+  if constexpr (V == 8 && sizeof(T) == 4) {
+    store_values<4>(p, v);
+    store_values<4>(p + 4, v + 4);
+  } else if constexpr (V == 8) {
+    *reinterpret_cast<uint4*>(p) = uint4{word(v[0], v[1]), word(v[2], v[3]), word(v[4], v[5]), word(v[6], v[7])};
+  } else if constexpr (V == 4 && sizeof(T) == 4) {
     *reinterpret_cast<float4*>(p) = float4{v[0], v[1], v[2], v[3]};
   } else if constexpr (V == 4) {
-    const auto word = [](float lo, float hi) {
-      return static_cast<uint32_t>(__builtin_bit_cast(uint16_t, static_cast<bf16_t>(lo))) |
-             (static_cast<uint32_t>(__builtin_bit_cast(uint16_t, static_cast<bf16_t>(hi))) << 16);
-    };
     *reinterpret_cast<uint2*>(p) = uint2{word(v[0], v[1]), word(v[2], v[3])};
   } else {
 #pragma unroll
@@ -937,19 +950,17 @@ __global__ void route_scale_bf16x8_kernel(bf16_t* __restrict__ hidden, int64_t l
 // (E x F), then every expert's up columns; `slices` partial sums lie `stride` elements apart. For the expert e that owns
 // column c, chosen by the row with weight w: g and u times w if `on_input`, clamped if limit > 0 (g from above, u on both
 // sides), hidden = g * sigmoid(slope * g) * (u + up_shift), times w unless `on_input`; zero if the row did not choose e.
-// V columns a thread (V > 1: F a multiple of V, 16-byte aligned rows).
+// V columns a thread (V > 1: F a multiple of V, rows aligned to V values). blockIdx.y walks the rows, so a row's choice is
+// the same for the whole block and is read once; blockIdx.x and the thread give the columns.
 template <int V, typename X, typename O>
 __global__ void route_glu_kernel(const X* __restrict__ gate_up, int64_t ld, int slices, int64_t stride,
                                  const int32_t* __restrict__ experts, const float* __restrict__ gates, int top, int F,
                                  int width, float limit, float slope, float up_shift, int on_input, O* __restrict__ out,
                                  int64_t T) {
-  const int pieces = width / V;
-  const int64_t total = T * pieces;
-  for (int64_t it = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; it < total;
-       it += static_cast<int64_t>(gridDim.x) * blockDim.x) {
-    const int64_t t = it / pieces;
-    const int c = V * static_cast<int>(it % pieces);
-    const int e = c / F;
+  const int c = V * static_cast<int>(blockIdx.x * blockDim.x + threadIdx.x);
+  if (c >= width) return;
+  const int e = c / F;
+  for (int64_t t = blockIdx.y; t < T; t += gridDim.y) {
     float w = 0.f;
     bool chosen = false;
     for (int k = 0; k < top; ++k)
@@ -1216,15 +1227,18 @@ extern "C" int distie_route_glu(const void* gate_up, int dtype, int64_t ld, int 
     return DISTIE_BAD_ARGUMENT;
   const int width = E * F;
   const int64_t stride = static_cast<int64_t>(T) * ld;
-  const bool wide = F % 4 == 0 && ld % 4 == 0 && reinterpret_cast<uintptr_t>(gate_up) % 16 == 0 &&
-                    reinterpret_cast<uintptr_t>(out) % 16 == 0;
-  const int64_t items = static_cast<int64_t>(T) * (wide ? width / 4 : width);
-  const int blocks = static_cast<int>(items / 256 + 1 < 16384 ? items / 256 + 1 : 16384);
+  const bool aligned = reinterpret_cast<uintptr_t>(gate_up) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0;
+  const int V = aligned && F % 8 == 0 && ld % 8 == 0 ? 8 : (aligned && F % 4 == 0 && ld % 4 == 0 ? 4 : 1);
+  const int per_row = width / V;
+  const int threads = per_row >= 256 ? 256 : (per_row > 64 ? 128 : 64);
+  const dim3 grid((per_row + threads - 1) / threads, T < 32768 ? T : 32768);
 #define DISTIE_ROUTE_GLU(V)                                                                                           \
-  DISTIE_DISPATCH(dtype, X, DISTIE_DISPATCH(out_dtype, O, (route_glu_kernel<V, X, O><<<blocks, 256, 0, stream>>>(     \
+  DISTIE_DISPATCH(dtype, X, DISTIE_DISPATCH(out_dtype, O, (route_glu_kernel<V, X, O><<<grid, threads, 0, stream>>>(   \
       static_cast<const X*>(gate_up), ld, slices, stride, experts, gates, top, F, width, limit, slope, up_shift,      \
       on_input, static_cast<O*>(out), T))))
-  if (wide) {
+  if (V == 8) {
+    DISTIE_ROUTE_GLU(8);
+  } else if (V == 4) {
     DISTIE_ROUTE_GLU(4);
   } else {
     DISTIE_ROUTE_GLU(1);

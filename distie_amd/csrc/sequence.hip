@@ -580,8 +580,12 @@ __global__ void causal_conv_bf16x8_kernel(const bf16_t* __restrict__ x, int64_t 
 // single dimensions). The blocks behind them: v for 16 tokens each; a thread owns one channel of v and, where
 // the 16 tokens lie side by side in one page, writes their values as one run of 32 bytes (the cache keeps v with
 // the key index innermost).
+// NORM: every q and k head first goes through x / sqrt(mean(x^2) + norm_eps) * weight over its D values (behind the
+// convolution, in front of the rotation): a first walk over the items leaves each item's sum of squares in LDS, and
+// an item of the second walk adds up those of its head, in their order.
 constexpr int VGROUP = 16;
 
+template <bool NORM>
 __global__ void conv_rope_kv_write_bf16_kernel(const bf16_t* __restrict__ product, int64_t ld, const bf16_t* __restrict__ weight,
                                                int taps, float* __restrict__ state, const float2* __restrict__ table,
                                                int pairs, float magnitude, bf16_t* __restrict__ q_out,
@@ -590,7 +594,10 @@ __global__ void conv_rope_kv_write_bf16_kernel(const bf16_t* __restrict__ produc
                                                const int32_t* __restrict__ token_request,
                                                const int32_t* __restrict__ state_slots, int T, int H, int G, int D, int E,
                                                int DP, int block_size, int has_kv, int write,
-                                               const int32_t* __restrict__ positions, float temp_coef, int temp_every) {
+                                               const int32_t* __restrict__ positions, float temp_coef, int temp_every,
+                                               const float* __restrict__ q_norm, const float* __restrict__ k_norm,
+                                               float norm_eps) {
+  extern __shared__ float squares[];                     // NORM: [heads of q and k, items of a head]
   const int N = H * D + (has_kv ? G * (D + E) : 0);
   if (static_cast<int>(blockIdx.x) >= T) {
     // ---- v: 16 tokens, one channel a thread
@@ -662,6 +669,24 @@ __global__ void conv_rope_kv_write_bf16_kernel(const bf16_t* __restrict__ produc
   const float qt = query_temperature(positions, t, temp_coef, temp_every);
   const int pair8 = pairs / 8, rest8 = (DP - 2 * pairs) / 8;
   const int per_head = pair8 + rest8;
+  if constexpr (NORM) {
+    for (int item = threadIdx.x; item < turned * per_head; item += blockDim.x) {
+      const int j8 = item % per_head;
+      const int base = item / per_head * D;
+      const int d0 = j8 < pair8 ? 8 * j8 : 2 * pairs + 8 * (j8 - pair8);
+      float x[8] = {}, self[8], sq = 0.f;
+      if (d0 < D) conv8(product, ld, own, weight, taps, t, i, base + d0, N, x, self);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) sq += x[e] * x[e];
+      if (j8 < pair8) {
+        conv8(product, ld, own, weight, taps, t, i, base + d0 + pairs, N, x, self);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) sq += x[e] * x[e];
+      }
+      squares[item] = sq;
+    }
+    __syncthreads();
+  }
   for (int item = threadIdx.x; item < turned * per_head; item += blockDim.x) {
     const int head = item / per_head;
     const int j8 = item % per_head;
@@ -669,11 +694,25 @@ __global__ void conv_rope_kv_write_bf16_kernel(const bf16_t* __restrict__ produc
     bf16_t* dst = head < H ? q_out + (t * H + head) * DP
                            : k_cache + ((page * G + (head - H)) * block_size + offset) * DP;
     const bool store = head < H || write;
+    const float* norm_weight = nullptr;
+    float r = 1.f;
+    if constexpr (NORM) {
+      norm_weight = head < H ? q_norm : k_norm;
+      if (norm_weight != nullptr) {
+        float total = 0.f;
+        for (int k = 0; k < per_head; ++k) total += squares[head * per_head + k];
+        r = 1.f / sqrtf(total / D + norm_eps);
+      }
+    }
     if (j8 < pair8) {
       const int d0 = 8 * j8, d1 = d0 + pairs;
       float x0[8], x1[8], s0[8], s1[8], a[8], c[8];
       conv8(product, ld, own, weight, taps, t, i, base + d0, N, x0, s0);
       conv8(product, ld, own, weight, taps, t, i, base + d1, N, x1, s1);
+      if (norm_weight != nullptr) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x0[e] *= r * norm_weight[d0 + e], x1[e] *= r * norm_weight[d1 + e];
+      }
       const float4* angles = reinterpret_cast<const float4*>(table + t * pairs + d0);       // (cos, sin) x 8
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
@@ -701,6 +740,10 @@ __global__ void conv_rope_kv_write_bf16_kernel(const bf16_t* __restrict__ produc
       if (d0 < D) {
         conv8(product, ld, own, weight, taps, t, i, base + d0, N, a, s0);
         if (single) shift_state8(own, taps, base + d0, N, s0);
+        if (norm_weight != nullptr) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) a[e] *= r * norm_weight[d0 + e];
+        }
       }
       if (head < H) {
 #pragma unroll
@@ -1103,18 +1146,27 @@ extern "C" int distie_conv_rope_kv_write(const void* product, int dtype, int64_t
   if ((pairs > 0 && table == nullptr) || (taps > 1 && state == nullptr) || (taps >= 1 && weight == nullptr))
     return DISTIE_BAD_ARGUMENT;
   if (has_kv && write && (k_cache == nullptr || v_cache == nullptr || slots == nullptr)) return DISTIE_BAD_ARGUMENT;
-  if (q_norm == nullptr && k_norm == nullptr &&
+  const bool normed = q_norm != nullptr || k_norm != nullptr;
+  const int norm_items = (has_kv ? H + G : H) * ((DP - pairs) / 8);
+  if ((!normed || (static_cast<size_t>(norm_items) * sizeof(float) <= 48 * 1024 && D % 8 == 0)) &&
       dtype == DISTIE_BF16 && (weight == nullptr || w_dtype == DISTIE_BF16) && (!write || cache_dtype == DISTIE_BF16) &&
       T >= 32 && D % 8 == 0 && E % 8 == 0 && DP % 8 == 0 && pairs % 8 == 0 && ld % 8 == 0 &&
       reinterpret_cast<uintptr_t>(product) % 16 == 0 && reinterpret_cast<uintptr_t>(q_out) % 16 == 0 && reinterpret_cast<uintptr_t>(k_cache) % 16 == 0 && reinterpret_cast<uintptr_t>(v_cache) % 16 == 0 && reinterpret_cast<uintptr_t>(state) % 16 == 0 && reinterpret_cast<uintptr_t>(table) % 16 == 0) {
     const int items = (has_kv ? H + G : H) * ((DP - pairs) / 8);
     const int threads8 = items > 128 ? 256 : (items > 64 ? 128 : 64);
     const int v_blocks = has_kv && (write || taps > 1) ? (T + VGROUP - 1) / VGROUP * G : 0;
-    conv_rope_kv_write_bf16_kernel<<<T + v_blocks, threads8, 0, stream>>>(
-        static_cast<const bf16_t*>(product), ld, static_cast<const bf16_t*>(weight), taps, state,
-        static_cast<const float2*>(table), pairs, magnitude, static_cast<bf16_t*>(q_out), static_cast<bf16_t*>(k_cache),
-        static_cast<bf16_t*>(v_cache), slots, cu_q, token_request, state_slots, T, H, G, D, E, DP, block_size, has_kv, write,
-        positions, temp_coef, temp_every);
+#define DISTIE_CONV_ROPE_BF16(NORM, LDS)                                                                                 \
+    conv_rope_kv_write_bf16_kernel<NORM><<<T + v_blocks, threads8, LDS, stream>>>(                                        \
+        static_cast<const bf16_t*>(product), ld, static_cast<const bf16_t*>(weight), taps, state,                         \
+        static_cast<const float2*>(table), pairs, magnitude, static_cast<bf16_t*>(q_out), static_cast<bf16_t*>(k_cache),  \
+        static_cast<bf16_t*>(v_cache), slots, cu_q, token_request, state_slots, T, H, G, D, E, DP, block_size, has_kv,    \
+        write, positions, temp_coef, temp_every, q_norm, k_norm, norm_eps)
+    if (normed) {
+      DISTIE_CONV_ROPE_BF16(true, static_cast<size_t>(norm_items) * sizeof(float));
+    } else {
+      DISTIE_CONV_ROPE_BF16(false, 0);
+    }
+#undef DISTIE_CONV_ROPE_BF16
     return launch_status();
   }
   const int work = DP - pairs > E ? DP - pairs : E;

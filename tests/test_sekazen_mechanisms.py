@@ -84,11 +84,12 @@ def test_norm_around_one_and_the_branch_reads(ops, width):
         assert torch.equal(ops.dense(h).cpu(), residual.cpu().to(dtype))
 
 
-@pytest.mark.parametrize("dims,dim,scaling", [(8, 16, True), (16, 16, False), (6, 20, True), (2, 32, False), (64, 64, True)])
-def test_head_norm_and_banded_rotation(ops, dims, dim, scaling):
+@pytest.mark.parametrize("dims,dim,E,scaling", [(8, 16, 12, True), (16, 16, 16, False), (6, 20, 12, True), (2, 32, 8, False),
+                                                 (64, 64, 64, True), (32, 128, 128, True), (16, 64, 32, False)])
+def test_head_norm_and_banded_rotation(ops, dims, dim, E, scaling):
     """Behind the stacked product: the norm over every head of q and k (one weight for all heads, as stored), then
     the rotation of a head's first dimensions by frequencies in bands; values pass. Positions up to a few hundred."""
-    H, G, E, eps = 3, 1, 12, 1e-4
+    H, G, eps = 3, 1, 1e-4
     rot = {"base": 300.0, "dims": dims}
     if scaling:
         rot["scaling"] = {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 32}
@@ -99,7 +100,7 @@ def test_head_norm_and_banded_rotation(ops, dims, dim, scaling):
     lengths = (300, 5)
     for dtype in act_types(ops):
         wq, wk = (1 + rnd(dim, seed=1, scale=0.3)).float(), (1 + rnd(dim, seed=2, scale=0.3)).float()
-        seqs = [rnd(n, H * dim + G * (dim + E) + 3, seed=10 + i, scale=2.0).to(dtype) for i, n in enumerate(lengths)]
+        seqs = [rnd(n, H * dim + G * (dim + E) + (8 if dims % 16 == 0 else 3), seed=10 + i, scale=2.0).to(dtype) for i, n in enumerate(lengths)]
         needs = build_part("mixer", PartSpec("conv_gated_attention", "a.", {
             "hidden_size": 8, "num_heads": H, "num_kv_heads": G, "head_dim": dim, "value_dim": E, "conv_taps": 0,
             "window": None, "scale": 1.0})).cache_requirement()
