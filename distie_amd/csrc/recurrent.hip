@@ -842,20 +842,26 @@ __device__ __forceinline__ void unpack8(const uint4& raw, float v[8]) {
   }
 }
 
-__global__ void __launch_bounds__(256)
-route_topk_bf16_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ weight, const float* __restrict__ bias,
-                       int32_t* __restrict__ experts, float* __restrict__ gates, int C, int E, int top, int sigmoid) {
-  __shared__ float z[ROUTE_MAX_EXPERTS];
-  __shared__ float part[4][ROUTE_GROUP];
-  __shared__ float chosen[ROUTE_MAX_TOP];
-  const int64_t t = blockIdx.x;
+// One row's router by one block of 256 threads: the chosen experts (largest logit first) and their weights end up in
+// `ids` and `weights` (LDS), for every thread of the block to read.
+struct RouteScratch {
+  float z[ROUTE_MAX_EXPERTS];
+  float part[4][ROUTE_GROUP];
+  float chosen[ROUTE_MAX_TOP];
+  int ids[ROUTE_MAX_TOP];
+  float weights[ROUTE_MAX_TOP];
+};
+
+__device__ __forceinline__ void route_row_bf16(const bf16_t* __restrict__ x_row, const bf16_t* __restrict__ weight,
+                                               const float* __restrict__ bias, int C, int E, int top, int sigmoid,
+                                               RouteScratch& lds) {
   const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
   const int pieces = C / 8;
   for (int e0 = 0; e0 < E; e0 += ROUTE_GROUP) {
     float acc[ROUTE_GROUP] = {};
     for (int p = threadIdx.x; p < pieces; p += 256) {
       uint4 raw[ROUTE_GROUP];
-      const uint4 mine = *reinterpret_cast<const uint4*>(x + t * C + 8 * p);
+      const uint4 mine = *reinterpret_cast<const uint4*>(x_row + 8 * p);
 #pragma unroll
       for (int g = 0; g < ROUTE_GROUP; ++g)
         raw[g] = *reinterpret_cast<const uint4*>(weight + static_cast<int64_t>(min(e0 + g, E - 1)) * C + 8 * p);
@@ -872,38 +878,52 @@ route_topk_bf16_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ 
 #pragma unroll
     for (int g = 0; g < ROUTE_GROUP; ++g) {
       const float total = wave_sum(acc[g]);
-      if (lane == 0) part[wave][g] = total;
+      if (lane == 0) lds.part[wave][g] = total;
     }
     __syncthreads();
     if (threadIdx.x < ROUTE_GROUP && e0 + threadIdx.x < E) {
       const int e = e0 + threadIdx.x;
-      z[e] = part[0][threadIdx.x] + part[1][threadIdx.x] + part[2][threadIdx.x] + part[3][threadIdx.x] +
-             (bias != nullptr ? bias[e] : 0.f);
+      lds.z[e] = lds.part[0][threadIdx.x] + lds.part[1][threadIdx.x] + lds.part[2][threadIdx.x] + lds.part[3][threadIdx.x] +
+                 (bias != nullptr ? bias[e] : 0.f);
     }
     __syncthreads();
   }
-  if (wave != 0) return;
-  for (int k = 0; k < top; ++k) {
-    float best = -INFINITY;
-    int at = 0x7fffffff;
-    for (int e = lane; e < E; e += 64) {
-      const float v = z[e];
-      if (v > best || (v == best && e < at)) best = v, at = e;
-    }
+  if (wave == 0) {
+    for (int k = 0; k < top; ++k) {
+      float best = -INFINITY;
+      int at = 0x7fffffff;
+      for (int e = lane; e < E; e += 64) {
+        const float v = lds.z[e];
+        if (v > best || (v == best && e < at)) best = v, at = e;
+      }
 #pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-      const float other = __shfl_xor(best, o, 64);
-      const int other_at = __shfl_xor(at, o, 64);
-      if (other > best || (other == best && other_at < at)) best = other, at = other_at;
+      for (int o = 32; o > 0; o >>= 1) {
+        const float other = __shfl_xor(best, o, 64);
+        const int other_at = __shfl_xor(at, o, 64);
+        if (other > best || (other == best && other_at < at)) best = other, at = other_at;
+      }
+      if (at == 0x7fffffff) at = k;
+      if (lane == 0) {
+        lds.ids[k] = at;
+        lds.chosen[k] = best;
+      }
+      if (at % 64 == lane) lds.z[at] = -INFINITY;
     }
-    if (at == 0x7fffffff) at = k;
-    if (lane == 0) {
-      experts[t * top + k] = at;
-      chosen[k] = best;
-    }
-    if (at % 64 == lane) z[at] = -INFINITY;
+    if (lane == 0) write_route_weights(lds.chosen, lds.weights, top, sigmoid);
   }
-  if (lane == 0) write_route_weights(chosen, gates + t * top, top, sigmoid);
+  __syncthreads();
+}
+
+__global__ void __launch_bounds__(256)
+route_topk_bf16_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ weight, const float* __restrict__ bias,
+                       int32_t* __restrict__ experts, float* __restrict__ gates, int C, int E, int top, int sigmoid) {
+  __shared__ RouteScratch lds;
+  const int64_t t = blockIdx.x;
+  route_row_bf16(x + t * C, weight, bias, C, E, top, sigmoid, lds);
+  if (threadIdx.x < top) {
+    experts[t * top + threadIdx.x] = lds.ids[threadIdx.x];
+    gates[t * top + threadIdx.x] = lds.weights[threadIdx.x];
+  }
 }
 
 // hidden [T, ld]: the columns [e * F, (e + 1) * F) of expert e times the row's weight for e, zero if e was not chosen
@@ -952,6 +972,8 @@ __global__ void route_scale_bf16x8_kernel(bf16_t* __restrict__ hidden, int64_t l
 // sides), hidden = g * sigmoid(slope * g) * (u + up_shift), times w unless `on_input`; zero if the row did not choose e.
 // V columns a thread (V > 1: F a multiple of V, rows aligned to V values). blockIdx.y walks the rows, so a row's choice is
 // the same for the whole block and is read once; blockIdx.x and the thread give the columns.
+constexpr int GLU_ROWS = 4;
+
 template <int V, typename X, typename O>
 __global__ void route_glu_kernel(const X* __restrict__ gate_up, int64_t ld, int slices, int64_t stride,
                                  const int32_t* __restrict__ experts, const float* __restrict__ gates, int top, int F,
@@ -960,27 +982,81 @@ __global__ void route_glu_kernel(const X* __restrict__ gate_up, int64_t ld, int 
   const int c = V * static_cast<int>(blockIdx.x * blockDim.x + threadIdx.x);
   if (c >= width) return;
   const int e = c / F;
-  for (int64_t t = blockIdx.y; t < T; t += gridDim.y) {
-    float w = 0.f;
-    bool chosen = false;
-    for (int k = 0; k < top; ++k)
-      if (experts[t * top + k] == e) w = gates[t * top + k], chosen = true;
-    float h[V] = {};
-    if (chosen) {
-      float g[V], u[V];
-      sum_values<V>(gate_up + t * ld + c, slices, stride, g);
-      sum_values<V>(gate_up + t * ld + width + c, slices, stride, u);
+  // GLU_ROWS rows a block row: their choices first, then every chosen row's loads together, then the arithmetic
+  for (int64_t t0 = static_cast<int64_t>(blockIdx.y) * GLU_ROWS; t0 < T; t0 += static_cast<int64_t>(gridDim.y) * GLU_ROWS) {
+    float w[GLU_ROWS], g[GLU_ROWS][V], u[GLU_ROWS][V];
+    bool chosen[GLU_ROWS];
 #pragma unroll
-      for (int k = 0; k < V; ++k) {
-        float gk = g[k], uk = u[k];
-        if (on_input) gk *= w, uk *= w;
-        if (limit > 0.f) gk = fminf(gk, limit), uk = fminf(fmaxf(uk, -limit), limit);
-        h[k] = gk / (1.f + expf(-slope * gk)) * (uk + up_shift);
-        if (!on_input) h[k] *= w;
+    for (int r = 0; r < GLU_ROWS; ++r) {
+      w[r] = 0.f, chosen[r] = false;
+      const int64_t t = t0 + r;
+      if (t < T) {
+        for (int k = 0; k < top; ++k)
+          if (experts[t * top + k] == e) w[r] = gates[t * top + k], chosen[r] = true;
       }
     }
-    store_values<V>(out + t * width + c, h);
+#pragma unroll
+    for (int r = 0; r < GLU_ROWS; ++r) {
+      if (!chosen[r]) continue;
+      sum_values<V>(gate_up + (t0 + r) * ld + c, slices, stride, g[r]);
+      sum_values<V>(gate_up + (t0 + r) * ld + width + c, slices, stride, u[r]);
+    }
+#pragma unroll
+    for (int r = 0; r < GLU_ROWS; ++r) {
+      if (t0 + r >= T) break;
+      float h[V] = {};
+      if (chosen[r]) {
+#pragma unroll
+        for (int k = 0; k < V; ++k) {
+          float gk = g[r][k], uk = u[r][k];
+          if (on_input) gk *= w[r], uk *= w[r];
+          if (limit > 0.f) gk = fminf(gk, limit), uk = fminf(fmaxf(uk, -limit), limit);
+          h[k] = gk / (1.f + expf(-slope * gk)) * (uk + up_shift);
+          if (!on_input) h[k] *= w[r];
+        }
+      }
+      store_values<V>(out + (t0 + r) * width + c, h);
+    }
   }
+}
+
+// Router and hidden values in one launch, for steps of few rows (bfloat16 rows and router weights, C a multiple of 8):
+// every block works out its row's choice again (the row and the router's weights come from the cache) and then does
+// `route_glu_kernel`'s work on its 256 * V columns. blockIdx.y: the row.
+template <int V, typename X, typename O>
+__global__ void __launch_bounds__(256)
+route_topk_glu_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ weight, const float* __restrict__ bias, int C,
+                      int E, int top, int sigmoid, const X* __restrict__ gate_up, int64_t ld, int slices, int64_t stride,
+                      int F, int width, float limit, float slope, float up_shift, int on_input, O* __restrict__ out) {
+  __shared__ RouteScratch lds;
+  const int64_t t = blockIdx.y;
+  const int c = V * static_cast<int>(blockIdx.x * blockDim.x + threadIdx.x);
+  // the thread's columns are asked for before the choice is known (few rows: reading what is not chosen costs nothing
+  // beside the wait it saves)
+  float g[V] = {}, u[V] = {};
+  if (c < width) {
+    sum_values<V>(gate_up + t * ld + c, slices, stride, g);
+    sum_values<V>(gate_up + t * ld + width + c, slices, stride, u);
+  }
+  route_row_bf16(x + t * C, weight, bias, C, E, top, sigmoid, lds);
+  if (c >= width) return;
+  const int e = c / F;
+  float w = 0.f;
+  bool chosen = false;
+  for (int k = 0; k < top; ++k)
+    if (lds.ids[k] == e) w = lds.weights[k], chosen = true;
+  float h[V] = {};
+  if (chosen) {
+#pragma unroll
+    for (int k = 0; k < V; ++k) {
+      float gk = g[k], uk = u[k];
+      if (on_input) gk *= w, uk *= w;
+      if (limit > 0.f) gk = fminf(gk, limit), uk = fminf(fmaxf(uk, -limit), limit);
+      h[k] = gk / (1.f + expf(-slope * gk)) * (uk + up_shift);
+      if (!on_input) h[k] *= w;
+    }
+  }
+  store_values<V>(out + t * width + c, h);
 }
 
 // x <- cap * tanh(x / cap)
@@ -1231,7 +1307,8 @@ extern "C" int distie_route_glu(const void* gate_up, int dtype, int64_t ld, int 
   const int V = aligned && F % 8 == 0 && ld % 8 == 0 ? 8 : (aligned && F % 4 == 0 && ld % 4 == 0 ? 4 : 1);
   const int per_row = width / V;
   const int threads = per_row >= 256 ? 256 : (per_row > 64 ? 128 : 64);
-  const dim3 grid((per_row + threads - 1) / threads, T < 32768 ? T : 32768);
+  const int row_groups = (T + GLU_ROWS - 1) / GLU_ROWS;
+  const dim3 grid((per_row + threads - 1) / threads, row_groups < 32768 ? row_groups : 32768);
 #define DISTIE_ROUTE_GLU(V)                                                                                           \
   DISTIE_DISPATCH(dtype, X, DISTIE_DISPATCH(out_dtype, O, (route_glu_kernel<V, X, O><<<grid, threads, 0, stream>>>(   \
       static_cast<const X*>(gate_up), ld, slices, stride, experts, gates, top, F, width, limit, slope, up_shift,      \
@@ -1244,6 +1321,36 @@ extern "C" int distie_route_glu(const void* gate_up, int dtype, int64_t ld, int 
     DISTIE_ROUTE_GLU(1);
   }
 #undef DISTIE_ROUTE_GLU
+  return launch_status();
+}
+
+// `distie_route_topk` (bfloat16 rows and weights) and `distie_route_glu` in one launch; for steps of few rows.
+extern "C" int distie_route_topk_glu(const void* x, const void* weight, const float* bias, int C, int sigmoid,
+                                     const void* gate_up, int dtype, int64_t ld, int slices, int T, int top, int E, int F,
+                                     float limit, float slope, float up_shift, int on_input, void* out, int out_dtype,
+                                     hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (C < 8 || C % 8 || E < 1 || E > ROUTE_MAX_EXPERTS || top < 1 || top > E || top > ROUTE_MAX_TOP || F < 1 || slices < 1 ||
+      T > 65535 || (slices > 1 && dtype != DISTIE_F32) || ld < 2 * static_cast<int64_t>(E) * F ||
+      reinterpret_cast<uintptr_t>(x) % 16 != 0 || reinterpret_cast<uintptr_t>(weight) % 16 != 0)
+    return DISTIE_BAD_ARGUMENT;
+  const int width = E * F;
+  const int64_t stride = static_cast<int64_t>(T) * ld;
+  const bool aligned = reinterpret_cast<uintptr_t>(gate_up) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0;
+  const int V = aligned && F % 8 == 0 && ld % 8 == 0 ? 8 : (aligned && F % 4 == 0 && ld % 4 == 0 ? 4 : 1);
+  const dim3 grid((width / V + 255) / 256, T);
+#define DISTIE_ROUTE_TOPK_GLU(V)                                                                                          \
+  DISTIE_DISPATCH(dtype, X, DISTIE_DISPATCH(out_dtype, O, (route_topk_glu_kernel<V, X, O><<<grid, 256, 0, stream>>>(       \
+      static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(weight), bias, C, E, top, sigmoid,                        \
+      static_cast<const X*>(gate_up), ld, slices, stride, F, width, limit, slope, up_shift, on_input, static_cast<O*>(out)))))
+  if (V == 8) {
+    DISTIE_ROUTE_TOPK_GLU(8);
+  } else if (V == 4) {
+    DISTIE_ROUTE_TOPK_GLU(4);
+  } else {
+    DISTIE_ROUTE_TOPK_GLU(1);
+  }
+#undef DISTIE_ROUTE_TOPK_GLU
   return launch_status();
 }
 

@@ -268,7 +268,8 @@ __global__ void conv_rope_kv_write_kernel(const X* __restrict__ product, int64_t
                                           const int32_t* __restrict__ state_slots, int H, int G, int D, int E, int DP,
                                           int block_size, int has_kv, int write, const int32_t* __restrict__ positions,
                                           float temp_coef, int temp_every, const float* __restrict__ q_norm,
-                                          const float* __restrict__ k_norm, float norm_eps) {
+                                          const float* __restrict__ k_norm, float norm_eps, int slices, int64_t stride) {
+  // slices > 1 (taps 0 only): the product is partial sums that lie `stride` elements apart, added in order while read
   const int64_t t = blockIdx.x;
   const int head = blockIdx.y;
   const int N = H * D + (has_kv ? G * (D + E) : 0);
@@ -281,7 +282,8 @@ __global__ void conv_rope_kv_write_kernel(const X* __restrict__ product, int64_t
   const int64_t page = slot / block_size;
   const int offset = static_cast<int>(slot % block_size);
   auto value = [&](int c) {
-    const float self = to_float(product[t * ld + c]);
+    float self = to_float(product[t * ld + c]);
+    for (int s = 1; s < slices; ++s) self += to_float(product[s * stride + t * ld + c]);
     if (taps < 1) return self;
     float w[MAX_TAPS];
     for (int j = 0; j < taps; ++j) w[j] = to_float(weight[static_cast<int64_t>(c) * taps + j]);
@@ -585,6 +587,12 @@ __global__ void causal_conv_bf16x8_kernel(const bf16_t* __restrict__ x, int64_t 
 // an item of the second walk adds up those of its head, in their order.
 constexpr int VGROUP = 16;
 
+// eight float32 values from a 16-byte aligned place, two loads
+__device__ __forceinline__ void load_f32x8(const float* __restrict__ p, float v[8]) {
+  const float4 lo = reinterpret_cast<const float4*>(p)[0], hi = reinterpret_cast<const float4*>(p)[1];
+  v[0] = lo.x, v[1] = lo.y, v[2] = lo.z, v[3] = lo.w, v[4] = hi.x, v[5] = hi.y, v[6] = hi.z, v[7] = hi.w;
+}
+
 template <bool NORM>
 __global__ void conv_rope_kv_write_bf16_kernel(const bf16_t* __restrict__ product, int64_t ld, const bf16_t* __restrict__ weight,
                                                int taps, float* __restrict__ state, const float2* __restrict__ table,
@@ -710,8 +718,11 @@ __global__ void conv_rope_kv_write_bf16_kernel(const bf16_t* __restrict__ produc
       conv8(product, ld, own, weight, taps, t, i, base + d0, N, x0, s0);
       conv8(product, ld, own, weight, taps, t, i, base + d1, N, x1, s1);
       if (norm_weight != nullptr) {
+        float w0[8], w1[8];
+        load_f32x8(norm_weight + d0, w0);
+        load_f32x8(norm_weight + d1, w1);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) x0[e] *= r * norm_weight[d0 + e], x1[e] *= r * norm_weight[d1 + e];
+        for (int e = 0; e < 8; ++e) x0[e] *= r * w0[e], x1[e] *= r * w1[e];
       }
       const float4* angles = reinterpret_cast<const float4*>(table + t * pairs + d0);       // (cos, sin) x 8
 #pragma unroll
@@ -741,8 +752,10 @@ __global__ void conv_rope_kv_write_bf16_kernel(const bf16_t* __restrict__ produc
         conv8(product, ld, own, weight, taps, t, i, base + d0, N, a, s0);
         if (single) shift_state8(own, taps, base + d0, N, s0);
         if (norm_weight != nullptr) {
+          float w0[8];
+          load_f32x8(norm_weight + d0, w0);
 #pragma unroll
-          for (int e = 0; e < 8; ++e) a[e] *= r * norm_weight[d0 + e];
+          for (int e = 0; e < 8; ++e) a[e] *= r * w0[e];
         }
       }
       if (head < H) {
@@ -1133,7 +1146,8 @@ extern "C" int distie_conv_rope_kv_write(const void* product, int dtype, int64_t
                                          const int32_t* cu_q, const int32_t* token_request, const int32_t* state_slots,
                                          int T, int H, int G, int D, int E, int DP, int block_size, int has_kv, int write,
                                          const int32_t* positions, float temp_coef, int temp_every, const float* q_norm,
-                                         const float* k_norm, float norm_eps, hipStream_t stream) {
+                                         const float* k_norm, float norm_eps, int slices, int q_dtype, hipStream_t stream) {
+  // slices > 1: `product` is float32 partial sums [slices, T, ld] (no convolution then); q_out is of `q_dtype`
   // temp_every >= 1: q of the token at position p times 1 + temp_coef * ln(floor((p + 1) / temp_every) + 1)
   // q_norm / k_norm (float32 [D], null: none): every q / k head goes through x / sqrt(mean(x^2) + norm_eps) * weight
   // over its D values, behind the convolution and in front of the rotation
@@ -1146,14 +1160,19 @@ extern "C" int distie_conv_rope_kv_write(const void* product, int dtype, int64_t
   if ((pairs > 0 && table == nullptr) || (taps > 1 && state == nullptr) || (taps >= 1 && weight == nullptr))
     return DISTIE_BAD_ARGUMENT;
   if (has_kv && write && (k_cache == nullptr || v_cache == nullptr || slots == nullptr)) return DISTIE_BAD_ARGUMENT;
+  if (slices < 1 || (slices > 1 && (dtype != DISTIE_F32 || taps >= 1)) || (q_dtype != dtype && dtype != DISTIE_F32))
+    return DISTIE_BAD_ARGUMENT;
+  const int64_t stride = static_cast<int64_t>(T) * ld;
   const bool normed = q_norm != nullptr || k_norm != nullptr;
   const int norm_items = (has_kv ? H + G : H) * ((DP - pairs) / 8);
-  if ((!normed || (static_cast<size_t>(norm_items) * sizeof(float) <= 48 * 1024 && D % 8 == 0)) &&
-      dtype == DISTIE_BF16 && (weight == nullptr || w_dtype == DISTIE_BF16) && (!write || cache_dtype == DISTIE_BF16) &&
+  if ((!normed || (static_cast<size_t>(norm_items) * sizeof(float) <= 48 * 1024 && D % 8 == 0 && pairs % 4 == 0 &&
+                   reinterpret_cast<uintptr_t>(q_norm) % 16 == 0 && reinterpret_cast<uintptr_t>(k_norm) % 16 == 0)) &&
+      dtype == DISTIE_BF16 && q_dtype == DISTIE_BF16 && (weight == nullptr || w_dtype == DISTIE_BF16) && (!write || cache_dtype == DISTIE_BF16) &&
       T >= 32 && D % 8 == 0 && E % 8 == 0 && DP % 8 == 0 && pairs % 8 == 0 && ld % 8 == 0 &&
       reinterpret_cast<uintptr_t>(product) % 16 == 0 && reinterpret_cast<uintptr_t>(q_out) % 16 == 0 && reinterpret_cast<uintptr_t>(k_cache) % 16 == 0 && reinterpret_cast<uintptr_t>(v_cache) % 16 == 0 && reinterpret_cast<uintptr_t>(state) % 16 == 0 && reinterpret_cast<uintptr_t>(table) % 16 == 0) {
     const int items = (has_kv ? H + G : H) * ((DP - pairs) / 8);
-    const int threads8 = items > 128 ? 256 : (items > 64 ? 128 : 64);
+    // with head norms a thread walks its items twice: as many threads as items (up to 512), so that it has one
+    const int threads8 = normed && items <= 512 ? (items + 63) / 64 * 64 : (items > 128 ? 256 : (items > 64 ? 128 : 64));
     const int v_blocks = has_kv && (write || taps > 1) ? (T + VGROUP - 1) / VGROUP * G : 0;
 #define DISTIE_CONV_ROPE_BF16(NORM, LDS)                                                                                 \
     conv_rope_kv_write_bf16_kernel<NORM><<<T + v_blocks, threads8, LDS, stream>>>(                                        \
@@ -1173,12 +1192,23 @@ extern "C" int distie_conv_rope_kv_write(const void* product, int dtype, int64_t
   const int threads = work > 128 ? 256 : (work > 64 ? 128 : 64);
   const dim3 grid(T, has_kv ? H + 2 * G : H);
   if (weight == nullptr) w_dtype = dtype;
+  if (q_dtype != dtype) {
+    // a float32 product (partial sums or not) behind a model that computes in bfloat16: no filter, q in `q_dtype`
+    if (taps >= 1) return DISTIE_BAD_ARGUMENT;
+    DISTIE_DISPATCH(q_dtype, Q, DISTIE_DISPATCH(cache_dtype, C,
+        conv_rope_kv_write_kernel<float, float, Q, C><<<grid, threads, 0, stream>>>(
+            static_cast<const float*>(product), ld, nullptr, taps, state, static_cast<const float2*>(table),
+            pairs, magnitude, static_cast<Q*>(q_out), static_cast<C*>(k_cache), static_cast<C*>(v_cache), slots, cu_q,
+            token_request, state_slots, H, G, D, E, DP, block_size, has_kv, write, positions, temp_coef, temp_every,
+            q_norm, k_norm, norm_eps, slices, stride)));
+    return launch_status();
+  }
   DISTIE_DISPATCH(dtype, X, DISTIE_DISPATCH(w_dtype, W, DISTIE_DISPATCH(cache_dtype, C,
       conv_rope_kv_write_kernel<X, W, X, C><<<grid, threads, 0, stream>>>(
           static_cast<const X*>(product), ld, static_cast<const W*>(weight), taps, state, static_cast<const float2*>(table),
           pairs, magnitude, static_cast<X*>(q_out), static_cast<C*>(k_cache), static_cast<C*>(v_cache), slots, cu_q,
           token_request, state_slots, H, G, D, E, DP, block_size, has_kv, write, positions, temp_coef, temp_every,
-          q_norm, k_norm, norm_eps))));
+          q_norm, k_norm, norm_eps, slices, stride))));
   return launch_status();
 }
 

@@ -308,7 +308,7 @@ class HipOps(Ops):
         o.distie_causal_conv.argtypes = [_P, _I, _L, _P, _I, _I, _P, _P, _I, _L, _I, _P, _P, _P, _P, _I, _I, _P]
         o.distie_conv_state.argtypes = [_P, _I, _L, _I, _P, _P, _P, _I, _I, _I, _P]
         o.distie_conv_rope_kv_write.argtypes = [_P, _I, _L, _P, _I, _I, _P, _P, _I, _F, _P, _P, _P, _I, _P, _P, _P, _P,
-                                                _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _F, _I, _P, _P, _F, _P]
+                                                _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _F, _I, _P, _P, _F, _I, _I, _P]
         o.distie_sigmoid_gate.argtypes = [_P, _I, _I, _I, _P, _I, _L, _P, _I, _I, _I, _P]
         o.distie_rmsnorm_gate.argtypes = [_P, _P, _I, _F, _P, _I, _L, _P, _I, _I, _I, _I, _I, _P]
         o.distie_norm_chain.argtypes = [_P, _I, _I, _P, _P, _I, _I, _P, _F, _F, _P, _F, _P, _P, _F, _P, _I, _P, _I, _I, _P]
@@ -319,6 +319,7 @@ class HipOps(Ops):
         o.distie_lru_scan_chunked.argtypes = [_P, _P, _P, _P, _P, _P, _P, _I, _L, _I, _P, _I, _P, _P, _P, _I, _I, _I, _P]
         o.distie_route_topk.argtypes = [_P, _I, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _P]
         o.distie_route_glu.argtypes = [_P, _I, _L, _I, _P, _P, _I, _I, _I, _I, _F, _F, _F, _I, _P, _I, _P]
+        o.distie_route_topk_glu.argtypes = [_P, _P, _P, _I, _I, _P, _I, _L, _I, _I, _I, _I, _I, _F, _F, _F, _I, _P, _I, _P]
         o.distie_softcap_f32.argtypes = [_P, _L, _F, _P]
         o.distie_route_scale.argtypes = [_P, _I, _L, _P, _P, _I, _I, _I, _I, _P]
         o.distie_scale_f32.argtypes = [_P, _L, _F, _P]
@@ -1146,7 +1147,13 @@ class HipOps(Ops):
 
     def conv_rope_kv_write(self, product, conv_weight, state, meta, group, k_cache, v_cache, inv_freq, magnitude,
                            num_heads, num_kv_heads, dim, value_dim, padded_dim, has_kv, write, q_temp=None, qk_norm=None):
-        product = self.dense(product)
+        # without a filter the kernel adds up a product's partial sums itself while it reads them
+        slices, q_dtype = 1, None
+        if isinstance(product, PartialSums) and conv_weight is None:
+            slices, q_dtype, product = product.slices, product.dtype, product.data.view(-1, product.data.shape[-1])
+        else:
+            product = self.dense(product)
+            q_dtype = product.dtype
         q_norm = k_norm = None
         norm_eps = 0.0
         if qk_norm is not None:
@@ -1158,7 +1165,7 @@ class HipOps(Ops):
             if q_norm is None or (has_kv and k_norm is None):
                 raise KernelError("conv_rope_kv_write: a norm on the heads needs a weight for q, and for k where there are keys")
         self._own(product, conv_weight, state, k_cache, v_cache, inv_freq)
-        T, W = product.shape
+        T, W = product.shape[0] // slices, product.shape[1]
         channels = num_heads * dim + (num_kv_heads * (dim + value_dim) if has_kv else 0)
         taps = 0 if conv_weight is None else conv_weight.shape[1]
         if T != meta.num_tokens or W < channels:
@@ -1173,7 +1180,7 @@ class HipOps(Ops):
                 raise KernelError("conv_rope_kv_write: keys and values are cached in one dtype")
         pairs = 0 if inv_freq is None else inv_freq.shape[0]
         table = self._rope_table(meta, inv_freq) if pairs else None
-        q = torch.empty((T, num_heads * padded_dim), dtype=product.dtype, device=self.device)
+        q = torch.empty((T, num_heads * padded_dim), dtype=q_dtype, device=self.device)
         ptr = lambda t: t.data_ptr() if t is not None else None
         _check(self._ops.distie_conv_rope_kv_write(
             product.data_ptr(), _code(product), W, ptr(conv_weight), _code(conv_weight) if conv_weight is not None else _F32,
@@ -1183,7 +1190,7 @@ class HipOps(Ops):
             meta.state_slots.data_ptr(), T, num_heads, num_kv_heads, dim, value_dim, padded_dim, meta.block_size,
             1 if has_kv else 0, 1 if write else 0, meta.positions.data_ptr(), float(q_temp[0]) if q_temp else 0.0,
             int(q_temp[1]) if q_temp else 0, ptr(q_norm), ptr(k_norm) if has_kv else None, float(norm_eps),
-            self._stream()), "conv_rope_kv_write")
+            slices, _CODES[q_dtype], self._stream()), "conv_rope_kv_write")
         if taps > 1:
             if not meta.all_decode:
                 # (requests that bring one row had their state moved on by the kernel above)
@@ -1510,6 +1517,38 @@ class HipOps(Ops):
                                           gates.data_ptr(), T, top, num_experts, width, float(limit or 0.0), float(slope),
                                           float(up_shift), 1 if on_input else 0, out.data_ptr(), _code(out),
                                           self._stream()), "route_glu")
+        return out
+
+    FUSED_ROUTE_ROWS = 64       # up to so many rows every block works out its row's choice itself
+
+    def route_experts_glu(self, x, router_weight, router_bias, top, scoring, gate_up, num_experts, width, limit, slope,
+                          up_shift, on_input):
+        if scoring not in ("softmax", "sigmoid"):
+            raise KernelError(f"route_experts_glu: no scoring named {scoring!r}")
+        x = self.dense(x)
+        T, C = x.shape
+        if T > self.FUSED_ROUTE_ROWS or x.dtype != torch.bfloat16 or router_weight.dtype != torch.bfloat16 or C % 8 or \
+                x.data_ptr() % 16 or router_weight.data_ptr() % 16 or not x.is_contiguous():
+            return super().route_experts_glu(x, router_weight, router_bias, top, scoring, gate_up, num_experts, width,
+                                             limit, slope, up_shift, on_input)
+        if isinstance(gate_up, (PendingNorm, PendingProduct)):
+            gate_up = self.dense(gate_up)
+        slices, source, dtype = 1, gate_up, gate_up.dtype
+        if isinstance(gate_up, PartialSums):
+            slices, source = gate_up.slices, gate_up.data
+        self._own(x, router_weight, router_bias, source)
+        if tuple(router_weight.shape) != (num_experts, C) or not 1 <= top <= num_experts or gate_up.shape[0] != T or \
+                gate_up.shape[1] != 2 * num_experts * width or \
+                (router_bias is not None and (router_bias.dtype != torch.float32 or tuple(router_bias.shape) != (num_experts,))):
+            raise KernelError("route_experts_glu: x [T, C], router [E, C], bias float32 [E], gate_up [T, 2 * E * width]")
+        if limit is not None and not limit > 0:
+            raise KernelError("route_experts_glu: the limit must be positive")
+        out = torch.empty((T, num_experts * width), dtype=dtype, device=self.device)
+        _check(self._ops.distie_route_topk_glu(
+            x.data_ptr(), router_weight.data_ptr(), router_bias.data_ptr() if router_bias is not None else None, C,
+            1 if scoring == "sigmoid" else 0, source.data_ptr(), _code(source), gate_up.shape[1], slices, T, int(top),
+            num_experts, width, float(limit or 0.0), float(slope), float(up_shift), 1 if on_input else 0, out.data_ptr(),
+            _code(out), self._stream()), "route_topk_glu")
         return out
 
     def softcap(self, x, cap):

@@ -348,6 +348,13 @@ class Ops(abc.ABC):
         -> act [T, num_experts * width], in float32 behind the product's rounding."""
         raise NotImplementedError(f"{type(self).__name__} has no routed feed-forward")
 
+    def route_experts_glu(self, x, router_weight: torch.Tensor, router_bias: Optional[torch.Tensor], top: int,
+                          scoring: str, gate_up, num_experts: int, width: int, limit: Optional[float], slope: float,
+                          up_shift: float, on_input: bool) -> torch.Tensor:
+        """`route_topk` of x, then `route_glu` of `gate_up` with what it chose; an implementation may fuse the two."""
+        experts, gates = self.route_topk(x, router_weight, router_bias, top, scoring)
+        return self.route_glu(gate_up, experts, gates, num_experts, width, limit, slope, up_shift, on_input)
+
     def softcap(self, x: torch.Tensor, cap: float) -> torch.Tensor:
         """float32 [R, N] (in place) -> cap * tanh(x / cap)."""
         raise NotImplementedError(f"{type(self).__name__} has no cap on values")

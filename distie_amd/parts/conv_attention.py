@@ -143,7 +143,9 @@ class ConvGatedAttention(Mixer):
         return classes[min(bisect.bisect_left(classes, longest), len(classes) - 1)]
 
     def forward(self, ops, x, ctx, cache, writes_cache: bool):
-        product = ops.dense(ops.linear(x, self.in_weight, self.in_bias))
+        product = ops.linear(x, self.in_weight, self.in_bias)
+        if self.output_gate or self.conv_taps:
+            product = ops.dense(product)            # the gate's columns are read here; a filter reads earlier rows
         k_cache, v_cache = cache["k"], cache["v"]
         state = cache["conv"] if self.conv_taps > 1 else None
         q = ops.conv_rope_kv_write(product, self.conv_weight, state, ctx.meta, cache.group, k_cache, v_cache,

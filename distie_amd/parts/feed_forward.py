@@ -151,12 +151,13 @@ class RoutedExperts(FeedForward):
 
     def forward(self, ops, x, ctx):
         x = ops.dense(x)
-        experts, gates = ops.route_topk(x, self.router_weight, self.router_bias, self.top, self.scoring)
         if not self.plain:
-            hidden = ops.route_glu(ops.linear(x, self.gate_up_weight), experts, gates, self.num_experts,
-                                   self.expert_size, self.limit if self.activation == "clamped_glu" else None,
-                                   self.slope, self.up_shift, self.weight_on == "input")
+            hidden = ops.route_experts_glu(x, self.router_weight, self.router_bias, self.top, self.scoring,
+                                           ops.linear(x, self.gate_up_weight), self.num_experts, self.expert_size,
+                                           self.limit if self.activation == "clamped_glu" else None, self.slope,
+                                           self.up_shift, self.weight_on == "input")
             return ops.linear(hidden, self.down_weight)
+        experts, gates = ops.route_topk(x, self.router_weight, self.router_bias, self.top, self.scoring)
         hidden = ops.dense(ops.linear_silu_mul(x, self.gate_up_weight))
         hidden = ops.route_scale(hidden, experts, gates, self.num_experts, self.expert_size)
         return ops.linear(hidden, self.down_weight)

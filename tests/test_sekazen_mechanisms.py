@@ -280,6 +280,13 @@ def test_router_scores(ops, experts, top, width):
             for t in range(T):
                 mine = got_e[t].cpu().tolist()
                 assert (2 not in mine) or (0 in mine and mine.index(0) < mine.index(2))
+        # the router and the experts' hidden values in one call give what the two calls give
+        ff = 8
+        gate_up = rnd(T, 2 * experts * ff, seed=3).to(dtype).to(ops.device)
+        apart = ops.route_glu(gate_up, got_e, got_w, experts, ff, 1.5, 1.702, 1.0, True)
+        at_once = ops.route_experts_glu(x.to(ops.device), w.to(ops.device), None, top, "sigmoid", gate_up, experts, ff,
+                                        1.5, 1.702, 1.0, True)
+        assert torch.equal(ops.dense(apart), ops.dense(at_once))
 
 
 @pytest.mark.parametrize("experts,top,ff,limit", [(6, 2, 24, 1.25), (1, 1, 8, 0.5), (5, 5, 10, 2.0), (3, 1, 7, 1.0)])
