@@ -852,23 +852,25 @@ struct RouteScratch {
   float weights[ROUTE_MAX_TOP];
 };
 
+template <int GROUP>                                   // experts worked on side by side: 16, or 8 where there are no more
 __device__ __forceinline__ void route_row_bf16(const bf16_t* __restrict__ x_row, const bf16_t* __restrict__ weight,
                                                const float* __restrict__ bias, int C, int E, int top, int sigmoid,
                                                RouteScratch& lds) {
+  static_assert(GROUP <= ROUTE_GROUP, "the scratch holds ROUTE_GROUP sums a wave");
   const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
   const int pieces = C / 8;
-  for (int e0 = 0; e0 < E; e0 += ROUTE_GROUP) {
-    float acc[ROUTE_GROUP] = {};
+  for (int e0 = 0; e0 < E; e0 += GROUP) {
+    float acc[GROUP] = {};
     for (int p = threadIdx.x; p < pieces; p += 256) {
-      uint4 raw[ROUTE_GROUP];
+      uint4 raw[GROUP];
       const uint4 mine = *reinterpret_cast<const uint4*>(x_row + 8 * p);
 #pragma unroll
-      for (int g = 0; g < ROUTE_GROUP; ++g)
+      for (int g = 0; g < GROUP; ++g)
         raw[g] = *reinterpret_cast<const uint4*>(weight + static_cast<int64_t>(min(e0 + g, E - 1)) * C + 8 * p);
       float xv[8];
       unpack8(mine, xv);
 #pragma unroll
-      for (int g = 0; g < ROUTE_GROUP; ++g) {
+      for (int g = 0; g < GROUP; ++g) {
         float wv[8];
         unpack8(raw[g], wv);
 #pragma unroll
@@ -876,12 +878,12 @@ __device__ __forceinline__ void route_row_bf16(const bf16_t* __restrict__ x_row,
       }
     }
 #pragma unroll
-    for (int g = 0; g < ROUTE_GROUP; ++g) {
+    for (int g = 0; g < GROUP; ++g) {
       const float total = wave_sum(acc[g]);
       if (lane == 0) lds.part[wave][g] = total;
     }
     __syncthreads();
-    if (threadIdx.x < ROUTE_GROUP && e0 + threadIdx.x < E) {
+    if (threadIdx.x < GROUP && e0 + threadIdx.x < E) {
       const int e = e0 + threadIdx.x;
       lds.z[e] = lds.part[0][threadIdx.x] + lds.part[1][threadIdx.x] + lds.part[2][threadIdx.x] + lds.part[3][threadIdx.x] +
                  (bias != nullptr ? bias[e] : 0.f);
@@ -919,7 +921,11 @@ route_topk_bf16_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ 
                        int32_t* __restrict__ experts, float* __restrict__ gates, int C, int E, int top, int sigmoid) {
   __shared__ RouteScratch lds;
   const int64_t t = blockIdx.x;
-  route_row_bf16(x + t * C, weight, bias, C, E, top, sigmoid, lds);
+  if (E <= 8) {
+    route_row_bf16<8>(x + t * C, weight, bias, C, E, top, sigmoid, lds);
+  } else {
+    route_row_bf16<ROUTE_GROUP>(x + t * C, weight, bias, C, E, top, sigmoid, lds);
+  }
   if (threadIdx.x < top) {
     experts[t * top + threadIdx.x] = lds.ids[threadIdx.x];
     gates[t * top + threadIdx.x] = lds.weights[threadIdx.x];
@@ -1038,7 +1044,11 @@ route_topk_glu_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w
     sum_values<V>(gate_up + t * ld + c, slices, stride, g);
     sum_values<V>(gate_up + t * ld + width + c, slices, stride, u);
   }
-  route_row_bf16(x + t * C, weight, bias, C, E, top, sigmoid, lds);
+  if (E <= 8) {
+    route_row_bf16<8>(x + t * C, weight, bias, C, E, top, sigmoid, lds);
+  } else {
+    route_row_bf16<ROUTE_GROUP>(x + t * C, weight, bias, C, E, top, sigmoid, lds);
+  }
   if (c >= width) return;
   const int e = c / F;
   float w = 0.f;
