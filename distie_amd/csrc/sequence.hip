@@ -767,6 +767,109 @@ __global__ void conv_rope_kv_write_bf16_kernel(const bf16_t* __restrict__ produc
   }
 }
 
+// The same work for steps with head norms and no filter, a run of lanes a (token, q or k head): a lane owns eight
+// neighbouring dimensions (D a multiple of 8, DP at most 512), the head's sum of squares is a sum over its lanes, and a
+// lane gets the other half of its pairs from the lane pairs / 8 away. One walk over the values, no barrier. The blocks from
+// `qk_blocks` on write v: 16 tokens each, one channel a thread, as above.
+__global__ void __launch_bounds__(256)
+head_norm_rope_kv_write_bf16_kernel(const bf16_t* __restrict__ product, int64_t ld, const float2* __restrict__ table,
+                                    int pairs, float magnitude, bf16_t* __restrict__ q_out, bf16_t* __restrict__ k_cache,
+                                    bf16_t* __restrict__ v_cache, const int32_t* __restrict__ slots, int T, int H, int G,
+                                    int D, int E, int DP, int block_size, int has_kv, int write,
+                                    const int32_t* __restrict__ positions, float temp_coef, int temp_every,
+                                    const float* __restrict__ q_norm, const float* __restrict__ k_norm, float norm_eps,
+                                    int qk_blocks, int lanes) {
+  if (static_cast<int>(blockIdx.x) >= qk_blocks) {
+    const int t0 = (static_cast<int>(blockIdx.x) - qk_blocks) / G * VGROUP;
+    const int g = (static_cast<int>(blockIdx.x) - qk_blocks) % G;
+    const int n = min(VGROUP, T - t0);
+    const int64_t slot0 = slots[t0];
+    bool together = n == VGROUP && block_size % 8 == 0 && slot0 % block_size % 8 == 0 &&
+                    slot0 % block_size + VGROUP <= block_size;
+#pragma unroll
+    for (int k = 1; k < VGROUP; ++k) together = together && slots[min(t0 + k, T - 1)] == slot0 + k;
+    const uint16_t* rows = reinterpret_cast<const uint16_t*>(product);
+    uint16_t* cache = reinterpret_cast<uint16_t*>(v_cache);
+    for (int e = threadIdx.x; e < E; e += blockDim.x) {
+      const int c = (H + G) * D + g * E + e;
+      uint32_t bits[VGROUP];
+#pragma unroll
+      for (int k = 0; k < VGROUP; ++k) bits[k] = k < n ? rows[static_cast<int64_t>(t0 + k) * ld + c] : 0u;
+      if (together) {
+        uint16_t* dst = cache + ((slot0 / block_size * G + g) * DP + e) * block_size + slot0 % block_size;
+        *reinterpret_cast<uint4*>(dst) = uint4{bits[0] | (bits[1] << 16), bits[2] | (bits[3] << 16),
+                                               bits[4] | (bits[5] << 16), bits[6] | (bits[7] << 16)};
+        *reinterpret_cast<uint4*>(dst + 8) = uint4{bits[8] | (bits[9] << 16), bits[10] | (bits[11] << 16),
+                                                   bits[12] | (bits[13] << 16), bits[14] | (bits[15] << 16)};
+      } else {
+#pragma unroll
+        for (int k = 0; k < VGROUP; ++k) {
+          if (k >= n) break;
+          const int64_t slot = slots[t0 + k];
+          cache[((slot / block_size * G + g) * DP + e) * block_size + slot % block_size] = static_cast<uint16_t>(bits[k]);
+        }
+      }
+    }
+    return;
+  }
+  // `lanes` (a power of two, DP / 8 rounded up) lanes a head, 64 / lanes heads a wave
+  const int turned = has_kv ? H + G : H;
+  const int lane = threadIdx.x % 64 % lanes;
+  const int64_t unit = (static_cast<int64_t>(blockIdx.x) * 4 + threadIdx.x / 64) * (64 / lanes) + threadIdx.x % 64 / lanes;
+  const int64_t t = min(unit, static_cast<int64_t>(T) * turned - 1) / turned;
+  const int head = static_cast<int>(min(unit, static_cast<int64_t>(T) * turned - 1) % turned);
+  const bool valid = unit < static_cast<int64_t>(T) * turned && (head < H || write);      // the others only take part in the shuffles
+  const int d0 = 8 * lane;
+  float x[8] = {};
+  if (valid && d0 < D) unpack_bf16x8(load16(product + t * ld + head * D + d0), x);
+  const float* norm_weight = head < H ? q_norm : k_norm;
+  float sq = 0.f;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) sq += x[e] * x[e];
+  for (int o = lanes / 2; o > 0; o >>= 1) sq += __shfl_xor(sq, o, 64);       // every lane of the wave, whatever its head
+  if (norm_weight != nullptr) {
+    const float r = 1.f / sqrtf(sq / D + norm_eps);
+    if (d0 < D) {
+      float w[8];
+      load_f32x8(norm_weight + d0, w);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) x[e] *= r * w[e];
+    }
+  }
+  const int shift = pairs / 8;                           // lanes [0, shift) hold the first halves, [shift, 2 shift) the second
+  const int partner = threadIdx.x % 64 - lane + (lane < shift ? lane + shift : (lane < 2 * shift ? lane - shift : lane));
+  float other[8], out[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) other[e] = __shfl(x[e], partner, 64);
+  if (!valid) return;
+  if (lane < 2 * shift) {
+    const bool first = lane < shift;
+    const float4* angles = reinterpret_cast<const float4*>(table + t * pairs + 8 * (first ? lane : lane - shift));
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const float4 cs = angles[e];
+      const float c0 = cs.x * magnitude, s0 = cs.y * magnitude, c1 = cs.z * magnitude, s1 = cs.w * magnitude;
+      // (u, v) -> (u cos - v sin, v cos + u sin): the first half holds u, the second v
+      out[2 * e] = first ? x[2 * e] * c0 - other[2 * e] * s0 : x[2 * e] * c0 + other[2 * e] * s0;
+      out[2 * e + 1] = first ? x[2 * e + 1] * c1 - other[2 * e + 1] * s1 : x[2 * e + 1] * c1 + other[2 * e + 1] * s1;
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) out[e] = x[e];
+  }
+  if (head < H) {
+    if (d0 >= DP) return;
+    const float qt = query_temperature(positions, t, temp_coef, temp_every);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) out[e] *= qt;
+    *reinterpret_cast<uint4*>(q_out + (t * H + head) * DP + d0) = pack_bf16x8(out);
+  } else if (d0 < D) {
+    const int64_t slot = slots[t];
+    bf16_t* dst = k_cache + ((slot / block_size * G + (head - H)) * block_size + slot % block_size) * DP;
+    *reinterpret_cast<uint4*>(dst + d0) = pack_bf16x8(out);
+  }
+}
+
 // out = x * sigmoid(gates), eight a thread
 __global__ void sigmoid_gate_bf16x8_kernel(const bf16_t* __restrict__ x, int ldh, int E, const bf16_t* __restrict__ gates,
                                            int64_t ldg, bf16_t* __restrict__ out, int width, int64_t T) {
@@ -1174,6 +1277,19 @@ extern "C" int distie_conv_rope_kv_write(const void* product, int dtype, int64_t
     // with head norms a thread walks its items twice: as many threads as items (up to 512), so that it has one
     const int threads8 = normed && items <= 512 ? (items + 63) / 64 * 64 : (items > 128 ? 256 : (items > 64 ? 128 : 64));
     const int v_blocks = has_kv && (write || taps > 1) ? (T + VGROUP - 1) / VGROUP * G : 0;
+    if (normed && taps == 0 && DP <= 512) {
+      const int64_t units = static_cast<int64_t>(T) * (has_kv ? H + G : H);
+      int lanes = 1;
+      while (8 * lanes < DP) lanes *= 2;
+      const int per_block = 4 * (64 / lanes);
+      const int qk_blocks = static_cast<int>((units + per_block - 1) / per_block);
+      const int v_only = has_kv && write ? (T + VGROUP - 1) / VGROUP * G : 0;
+      head_norm_rope_kv_write_bf16_kernel<<<qk_blocks + v_only, 256, 0, stream>>>(
+          static_cast<const bf16_t*>(product), ld, static_cast<const float2*>(table), pairs, magnitude,
+          static_cast<bf16_t*>(q_out), static_cast<bf16_t*>(k_cache), static_cast<bf16_t*>(v_cache), slots, T, H, G, D, E, DP,
+          block_size, has_kv, write, positions, temp_coef, temp_every, q_norm, k_norm, norm_eps, qk_blocks, lanes);
+      return launch_status();
+    }
 #define DISTIE_CONV_ROPE_BF16(NORM, LDS)                                                                                 \
     conv_rope_kv_write_bf16_kernel<NORM><<<T + v_blocks, threads8, LDS, stream>>>(                                        \
         static_cast<const bf16_t*>(product), ld, static_cast<const bf16_t*>(weight), taps, state,                         \
