@@ -985,7 +985,13 @@ __global__ void route_glu_kernel(const X* __restrict__ gate_up, int64_t ld, int 
                                  const int32_t* __restrict__ experts, const float* __restrict__ gates, int top, int F,
                                  int width, float limit, float slope, float up_shift, int on_input, O* __restrict__ out,
                                  int64_t T) {
-  const int c = V * static_cast<int>(blockIdx.x * blockDim.x + threadIdx.x);
+  // Blocks go to the chip's eight dies in turn by their number (blockIdx.x fastest): with the columns taken from
+  // blockIdx.x alone, the blocks of one expert's columns would all land on the same die, and where most rows choose the
+  // same experts two dies would do the reading for all. The block row shifts the columns, so every die gets its share.
+  // A block's waves take runs of columns that lie a whole row of blocks apart, so a block meets several experts and has
+  // its share of the chosen ones.
+  const int column_block = (blockIdx.x + blockIdx.y) % gridDim.x;
+  const int c = V * static_cast<int>((threadIdx.x / 64 * gridDim.x + column_block) * 64 + threadIdx.x % 64);
   if (c >= width) return;
   const int e = c / F;
   // GLU_ROWS rows a block row: their choices first, then every chosen row's loads together, then the arithmetic

@@ -1502,10 +1502,17 @@ class HipOps(Ops):
     def route_glu(self, gate_up, experts, gates, num_experts, width, limit, slope, up_shift, on_input):
         if isinstance(gate_up, (PendingNorm, PendingProduct)):
             gate_up = self.dense(gate_up)
-        slices, source, dtype = 1, gate_up, gate_up.dtype
+        slices, source, dtype, ld = 1, gate_up, gate_up.dtype, gate_up.shape[1]
         if isinstance(gate_up, PartialSums):
             slices, source = gate_up.slices, gate_up.data
+        elif gate_up.dim() == 2 and gate_up.stride(1) == 1 and gate_up.stride(0) > gate_up.shape[1]:
+            # rows that lie further apart than they are wide (`linear_spread`): the kernel takes the row stride
+            ld = gate_up.stride(0)
+            if gate_up.device != self.device:
+                raise KernelError(f"tensor on {gate_up.device}, kernels run on {self.device}")
+            source = None
         self._own(source, experts, gates)
+        source = gate_up if source is None else source
         T, top = experts.shape
         if experts.dtype != torch.int32 or gates.dtype != torch.float32 or gates.shape != experts.shape or \
                 gate_up.shape[0] != T or gate_up.shape[1] != 2 * num_experts * width:
@@ -1513,7 +1520,7 @@ class HipOps(Ops):
         if limit is not None and not limit > 0:
             raise KernelError("route_glu: the limit must be positive")
         out = torch.empty((T, num_experts * width), dtype=dtype, device=self.device)
-        _check(self._ops.distie_route_glu(source.data_ptr(), _code(source), gate_up.shape[1], slices, experts.data_ptr(),
+        _check(self._ops.distie_route_glu(source.data_ptr(), _code(source), ld, slices, experts.data_ptr(),
                                           gates.data_ptr(), T, top, num_experts, width, float(limit or 0.0), float(slope),
                                           float(up_shift), 1 if on_input else 0, out.data_ptr(), _code(out),
                                           self._stream()), "route_glu")
