@@ -313,6 +313,12 @@ def test_clamped_gated_experts(ops, experts, top, ff, limit):
             got = ops.route_glu(gate_up.to(ops.device), chosen.to(torch.int32).to(ops.device), gates.to(ops.device),
                                 experts, ff, lim, slope, shift, on_input)
             close(ops.dense(got), want.view(T, -1), dtype, f"hidden values, on_input {on_input}, limit {lim}")
+            # rows that lie further apart than they are wide give the same
+            wide = torch.zeros(T, 2 * experts * ff + 24, dtype=dtype)
+            wide[:, :2 * experts * ff] = gate_up
+            spread = ops.route_glu(wide.to(ops.device)[:, :2 * experts * ff], chosen.to(torch.int32).to(ops.device),
+                                   gates.to(ops.device), experts, ff, lim, slope, shift, on_input)
+            assert torch.equal(ops.dense(spread), ops.dense(got))
         part = build_part("feed_forward", PartSpec("routed_experts", "m.", {
             "hidden_size": C, "num_experts": experts, "top": top, "expert_size": ff, "router_bias": False,
             "scoring": "sigmoid", "weight_on": "input", "activation": "clamped_glu", "limit": limit, "slope": 1.702,
