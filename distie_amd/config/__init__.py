@@ -1,6 +1,7 @@
 from .engine_config import EngineConfig, resolve_dtype
 from .model_config import (ConfigError, LayerCall, LayerSpec, ModelSpec, PartSpec, Qwen2Config,
                            read_config_json)
+from .dufelix_config import DufelixConfig
 from .duparax_config import DuparaxConfig
 from .musutar_config import MusutarConfig
 from .sekazen_config import SekazenConfig
@@ -9,6 +10,6 @@ from .registry import (architecture_of, config_from_dict, known_architectures, l
 
 __all__ = [
     "EngineConfig", "resolve_dtype", "ConfigError", "LayerCall", "LayerSpec", "ModelSpec", "PartSpec",
-    "Qwen2Config", "MusutarConfig", "DuparaxConfig", "SekazenConfig", "read_config_json", "architecture_of", "config_from_dict", "known_architectures",
+    "Qwen2Config", "MusutarConfig", "DuparaxConfig", "SekazenConfig", "DufelixConfig", "read_config_json", "architecture_of", "config_from_dict", "known_architectures",
     "load_model_config", "model_spec_from_dir", "register_architecture",
 ]

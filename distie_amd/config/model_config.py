@@ -39,10 +39,14 @@ class PartSpec:
 class LayerSpec:
     """A layer = an arrangement (`block`) and the parts it arranges, under the names that the block's
     class gives them (the pre-norm block of this package: `mixer`, `feed_forward`, `mixer_norm`,
-    `feed_forward_norm`; another block may arrange four norms, two mixers, or no feed-forward)."""
+    `feed_forward_norm`; another block may arrange four norms, two mixers, or no feed-forward).
+
+    `weights_of`: the layer is earlier layer j once more, with j's parts and tensors (the model builds no second copy of
+    them) but a cache and state of its own; `block` and `parts` then equal layer j's."""
 
     block: PartSpec
     parts: Mapping[str, PartSpec] = field(default_factory=dict)
+    weights_of: Optional[int] = None
 
 
 @dataclass(frozen=True)

@@ -11,6 +11,7 @@ from __future__ import annotations
 from typing import Any, Dict, Mapping
 
 from .model_config import ConfigError, ModelSpec, Qwen2Config, read_config_json
+from .dufelix_config import DufelixConfig
 from .duparax_config import DuparaxConfig
 from .musutar_config import MusutarConfig
 from .sekazen_config import SekazenConfig
@@ -73,3 +74,4 @@ register_architecture(Qwen2Config.architecture, Qwen2Config)
 register_architecture(MusutarConfig.architecture, MusutarConfig)
 register_architecture(DuparaxConfig.architecture, DuparaxConfig)
 register_architecture(SekazenConfig.architecture, SekazenConfig)
+register_architecture(DufelixConfig.architecture, DufelixConfig)

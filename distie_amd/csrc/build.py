@@ -36,7 +36,7 @@ HIP_FLAGS = ["-O3", f"--offload-arch={ARCH}", "-fPIC", "-std=c++17",
              "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option"]
 CXX_FLAGS = ["-O2", "-fPIC", "-std=c++17", "-pthread"]
 
-OPS_SOURCES = ["elementwise.hip", "gemm.hip", "gemv.hip", "decode_products.hip", "sampling.hip", "sequence.hip", "recurrent.hip"]
+OPS_SOURCES = ["elementwise.hip", "gemm.hip", "gemv.hip", "decode_products.hip", "sampling.hip", "sequence.hip", "recurrent.hip", "latent.hip", "ssm.hip"]
 ATTN_SOURCES = ["attention.hip"]
 LIBRARY_SOURCES = ["library_products.hip"]
 LINK_LIBS = {"library": ["-lhipblaslt"]}

@@ -16,6 +16,16 @@ constexpr int MAX_TAPS = 16;
 
 __device__ __forceinline__ float sigmoidf(float x) { return 1.f / (1.f + __expf(-x)); }
 __device__ __forceinline__ float siluf(float x) { return x / (1.f + __expf(-x)); }
+// kinds: 0 relu squared, 1 silu, 2 gelu (tanh form), 3 relu
+__device__ __forceinline__ float activate(float z, int kind) {
+  if (kind == 0) {
+    const float p = fmaxf(z, 0.f);
+    return p * p;
+  }
+  if (kind == 1) return z / (1.f + expf(-z));
+  if (kind == 2) return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+  return fmaxf(z, 0.f);
+}
 // a query temperature by position: 1 + coef * ln(floor((p + 1) / every) + 1); every < 1: none
 __device__ __forceinline__ float query_temperature(const int32_t* __restrict__ positions, int64_t t, float coef, int every) {
   if (every < 1) return 1.f;
@@ -219,8 +229,9 @@ __global__ void causal_conv_kernel(const X* __restrict__ x, int64_t ldx, const W
   for (int j = 0; j < taps; ++j) w[j] = to_float(weight[static_cast<int64_t>(c) * taps + j]);
   float acc = conv_at(x, ldx, own, w, taps, t, i, c, N);
   const float self = to_float(x[t * ldx + c]);
-  if (residual) acc += self;
+  if (residual & 1) acc += self;
   if (bias != nullptr) acc += bias[c];
+  if (residual >> 1) acc = activate(acc, (residual >> 1) - 1);       // an activation on the float32 sum
   out[t * ldo + c] = from_float<O>(acc);
   if (n == 1) {
     float keep[MAX_TAPS];
@@ -565,13 +576,17 @@ __global__ void causal_conv_bf16x8_kernel(const bf16_t* __restrict__ x, int64_t 
   float* own = state + static_cast<int64_t>(state_slots[b]) * (taps - 1) * N;
   float acc[8], self[8];
   conv8(x, ldx, own, weight, taps, t, i, c0, N, acc, self);
-  if (residual) {
+  if (residual & 1) {
 #pragma unroll
     for (int e = 0; e < 8; ++e) acc[e] += self[e];
   }
   if (bias != nullptr) {
 #pragma unroll
     for (int e = 0; e < 8; ++e) acc[e] += bias[c0 + e];
+  }
+  if (residual >> 1) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = activate(acc[e], (residual >> 1) - 1);
   }
   *reinterpret_cast<uint4*>(out + t * ldo + c0) = pack_bf16x8(acc);
   if (cu_q[b + 1] - first == 1 && taps > 1) shift_state8(own, taps, c0, N, self);
@@ -1208,12 +1223,15 @@ extern "C" int distie_hyper_step(float* streams, int S, const float* init, const
   return launch_status();
 }
 
+// `residual`: bit 0: the input itself is added; the bits above it: 1 + the kind of an activation on the sum (0: none)
 extern "C" int distie_causal_conv(const void* x, int x_dtype, int64_t ldx, const void* weight, int w_dtype, int taps,
                                   float* state, void* out, int out_dtype, int64_t ldo, int residual, const float* bias,
                                   const int32_t* cu_q, const int32_t* token_request, const int32_t* state_slots, int T,
                                   int N, hipStream_t stream) {
   if (T <= 0) return 0;
-  if (taps < 1 || taps > MAX_TAPS || N < 1 || ldx < N || ldo < N || (taps > 1 && state == nullptr)) return DISTIE_BAD_ARGUMENT;
+  if (taps < 1 || taps > MAX_TAPS || N < 1 || ldx < N || ldo < N || (taps > 1 && state == nullptr) || residual < 0 ||
+      (residual >> 1) > 4)
+    return DISTIE_BAD_ARGUMENT;
   if (x_dtype == DISTIE_BF16 && w_dtype == DISTIE_BF16 && out_dtype == DISTIE_BF16 && N % 8 == 0 && ldx % 8 == 0 &&
       ldo % 8 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0 && reinterpret_cast<uintptr_t>(state) % 16 == 0) {
     const int items = N / 8;

@@ -24,7 +24,20 @@ class Model:
     def __init__(self, spec: ModelSpec) -> None:
         self.spec = spec
         self.embed = build_part("embedding", spec.embedding)
-        self.blocks = [build_part("block", layer.block, layer.parts) for layer in spec.layers]
+        # a layer that uses an earlier layer's tensors is that layer's block once more: one set of parts and weights,
+        # and (the cache being declared and addressed by layer) pages and state of its own
+        self.blocks = []
+        for index, layer in enumerate(spec.layers):
+            if layer.weights_of is None:
+                self.blocks.append(build_part("block", layer.block, layer.parts))
+                continue
+            source = int(layer.weights_of)
+            if not 0 <= source < index or spec.layers[source].weights_of is not None:
+                raise ValueError(f"layer {index} uses the tensors of layer {source}, which must be an earlier layer with "
+                                 f"tensors of its own")
+            if (layer.block, dict(layer.parts)) != (spec.layers[source].block, dict(spec.layers[source].parts)):
+                raise ValueError(f"layer {index} uses the tensors of layer {source} and must be described like it")
+            self.blocks.append(self.blocks[source])
         self.final_norm = build_part("norm", spec.final_norm)
         self.position = build_part("position", spec.position) if spec.position is not None else None
         self.lm_head = build_part("head", spec.head)
@@ -37,8 +50,9 @@ class Model:
     def parts(self):
         """Every part of the model, in the order in which their tensors are declared."""
         yield from self.embed.parts()
-        for block in self.blocks:
-            yield from block.parts()
+        for index, block in enumerate(self.blocks):
+            if self.spec.layers[index].weights_of is None:
+                yield from block.parts()
         yield from self.final_norm.parts()
         if self.position is not None:
             yield from self.position.parts()

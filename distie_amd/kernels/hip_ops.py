@@ -326,6 +326,16 @@ class HipOps(Ops):
         o.distie_activation.argtypes = [_P, _I, _I, _P, _I, _L, _I, _P]
         o.distie_decay_scan.argtypes = [_P, _I, _L, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P]
         o.distie_decay_scan_chunked.argtypes = [_P, _I, _L, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]
+        o.distie_latent_norm_rope_write.argtypes = [_P, _L, _I, _P, _I, _P, _F, _I, _P, _F, _I, _P, _I, _P, _P, _I, _P,
+                                                    _I, _I, _I, _I, _P]
+        o.distie_rope_heads.argtypes = [_P, _I, _I, _I, _P, _I, _I, _I, _I, _I, _P, _F, _I, _P]
+        o.distie_heads_linear.argtypes = [_P, _I, _I, _P, _I, _P, _I, _I, _I, _I, _I, _P]
+        o.distie_head_gate.argtypes = [_P, _I, _I, _I, _P, _I, _L, _P, _I, _I, _I, _P]
+        o.distie_ssm_scan.argtypes = [_P, _I, _L, _P, _L, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]
+        o.distie_ssm_scan_chunked.argtypes = [_P, _I, _L, _P, _L, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I,
+                                              _I, _I, _P]
+        o.distie_gate_rmsnorm.argtypes = [_P, _P, _I, _F, _P, _I, _L, _P, _I, _I, _I, _I, _I, _P]
+        o.distie_glu_mul.argtypes = [_P, _I, _I, _P, _I, _I, _I, _I, _P]
         o.distie_argmax.argtypes = [_P, _P, _I, _I, _P, _P, _P]
         o.distie_argmax_parts.argtypes = [_I, _I]
         o.distie_sample.argtypes = [_P, _P, _P, _P, _P, _I, _I, _P, _P, _P, _P]
@@ -396,11 +406,13 @@ class HipOps(Ops):
                                             table.numel(), self._stream()), "scatter_i32")
         _mark_written(table)
 
-    def embed(self, ids, table):
+    def embed(self, ids, table, scale=1.0):
         self._own(ids, table)
         out = torch.empty((ids.shape[0], table.shape[1]), dtype=torch.float32, device=self.device)
         _check(self._ops.distie_embed(ids.data_ptr(), table.data_ptr(), _code(table), out.data_ptr(),
                                       ids.shape[0], table.shape[1], table.shape[0], self._stream()), "embed")
+        if scale != 1.0 and out.numel():
+            _check(self._ops.distie_scale_f32(out.data_ptr(), out.numel(), float(scale), self._stream()), "scale_f32")
         return out
 
     def _norm_later(self, residual, weight, out_dtype) -> bool:
@@ -1113,7 +1125,9 @@ class HipOps(Ops):
         _mark_written(streams)
         return streams, h
 
-    def causal_conv(self, x, weight, state, meta, residual=False, bias=None):
+    def causal_conv(self, x, weight, state, meta, residual=False, bias=None, act=None):
+        if act is not None and act not in self.ACTIVATIONS:
+            raise KernelError(f"causal_conv: no activation named {act!r}")
         x = self.dense(x)
         self._own(weight, state, bias)
         T, N = x.shape
@@ -1127,7 +1141,8 @@ class HipOps(Ops):
         out = torch.empty((T, N), dtype=x.dtype, device=self.device)
         _check(self._ops.distie_causal_conv(
             x_ptr, _code(x), ldx, weight.data_ptr(), _code(weight), taps, state.data_ptr() if taps > 1 else None,
-            out.data_ptr(), _code(out), N, 1 if residual else 0, bias.data_ptr() if bias is not None else None,
+            out.data_ptr(), _code(out), N, (1 if residual else 0) | (0 if act is None else (self.ACTIVATIONS[act] + 1) << 1),
+            bias.data_ptr() if bias is not None else None,
             meta.cu_q.data_ptr(), meta.token_request.data_ptr(), meta.state_slots.data_ptr(), T, N, self._stream()),
             "causal_conv")
         if taps > 1 and not meta.all_decode:
@@ -1200,12 +1215,20 @@ class HipOps(Ops):
             _mark_written(state)
         return q
 
-    def sigmoid_gate(self, x, num_heads, head_stride, width, gates):
+    def sigmoid_gate(self, x, num_heads, head_stride, width, gates, per_head=False):
         x = self.dense(x)
         self._own(x)
         T = x.shape[0]
         if x.shape[1] != num_heads * head_stride or width > head_stride:
             raise KernelError("sigmoid_gate: x must be [T, heads * head_stride]")
+        if per_head:
+            if gates is None:
+                raise KernelError("sigmoid_gate: a gate for each head needs the gates")
+            g_ptr, g_ld = self._rows_view(gates, num_heads)
+            out = torch.empty((T, num_heads * width), dtype=x.dtype, device=self.device)
+            _check(self._ops.distie_head_gate(x.data_ptr(), _code(x), head_stride, width, g_ptr, _code(gates), g_ld,
+                                              out.data_ptr(), _code(out), T, num_heads * width, self._stream()), "head_gate")
+            return out
         g_ptr, g_ld = self._rows_view(gates, num_heads * width) if gates is not None else (None, 0)
         out = torch.empty((T, num_heads * width), dtype=x.dtype, device=self.device)
         _check(self._ops.distie_sigmoid_gate(x.data_ptr(), _code(x), head_stride, width, g_ptr,
@@ -1267,10 +1290,25 @@ class HipOps(Ops):
         _mark_written(state)
         return out
 
-    def rmsnorm_gate(self, x, weight, eps, gates, out_dtype, group=None, gate="sigmoid"):
+    def rmsnorm_gate(self, x, weight, eps, gates, out_dtype, group=None, gate="sigmoid", gate_first=False):
         self._own(x, weight)
         if gate not in ("sigmoid", "silu"):
             raise KernelError(f"rmsnorm_gate: no gate named {gate!r}")
+        if gate_first or (group is not None and x.dim() == 2 and tuple(weight.shape) == (x.shape[1],) and group != x.shape[1]):
+            # the gate in front of the norm, every column with a weight of its own
+            if not gate_first or gates is None:
+                raise KernelError("rmsnorm_gate: a weight for every column of grouped norms goes with the gate in front")
+            if x.dtype != torch.float32 or x.dim() != 2 or tuple(weight.shape) != (x.shape[1],) or \
+                    (group is not None and (group < 1 or x.shape[1] % group)):
+                raise KernelError("rmsnorm_gate: x must be float32 [T, N], weight [N], N a multiple of the group")
+            T, N = x.shape
+            size = group or N
+            g_ptr, g_ld = self._rows_view(gates, N)
+            out = torch.empty((T, N), dtype=out_dtype, device=self.device)
+            _check(self._ops.distie_gate_rmsnorm(x.data_ptr(), weight.data_ptr(), _code(weight), float(eps), g_ptr,
+                                                 _code(gates), g_ld, out.data_ptr(), _code(out), T, size, N // size,
+                                                 1 if gate == "silu" else 0, self._stream()), "gate_rmsnorm")
+            return out
         if x.dtype != torch.float32 or x.dim() != 2 or (group is not None and (group < 1 or x.shape[1] % group)) or \
                 tuple(weight.shape) != (group or x.shape[1],):
             raise KernelError("rmsnorm_gate: x must be float32 [T, N], weight [N] (or [group], N a multiple of it)")
@@ -1590,6 +1628,124 @@ class HipOps(Ops):
         out = torch.empty(tuple(x.shape), dtype=dtype, device=self.device)
         _check(self._ops.distie_activation(source.data_ptr(), _code(source), slices, out.data_ptr(), _code(out), out.numel(),
                                            self.ACTIVATIONS[kind], self._stream()), "activation")
+        return out
+
+    # ---- a state with one decay a head and token, attention over a shared latent (csrc/ssm.hip, csrc/latent.hip)
+    SSM_CHUNKED_MIN_ROWS = 32        # a step with a portion of so many rows scans the state-space state in chunks
+
+    def ssm_scan(self, xbc, dt, dt_bias, a_log, skip, state, meta, num_heads, value_dim, state_size, groups):
+        xbc = self.dense(xbc)
+        H, P, N, G = num_heads, value_dim, state_size, groups
+        width = H * P + 2 * G * N
+        x_ptr, ld = self._rows_view(xbc, xbc.shape[1])
+        d_ptr, ldd = self._rows_view(dt, H)
+        self._own(dt_bias, a_log, skip, state)
+        T = xbc.shape[0]
+        if T != meta.num_tokens or xbc.shape[1] < width or dt.dtype != xbc.dtype or H % G:
+            raise KernelError("ssm_scan: x, B and C do not match the batch or the head counts")
+        if state.dtype != torch.float32 or tuple(state.shape[1:]) != (H, N, P):
+            raise KernelError("ssm_scan: the state is float32 [slots, heads, state_size, value_dim]")
+        for vector in (dt_bias, a_log, skip):
+            if vector.dtype != torch.float32 or tuple(vector.shape) != (H,):
+                raise KernelError("ssm_scan: dt_bias, a_log and skip are float32 [heads]")
+        out = torch.empty((T, H * P), dtype=torch.float32, device=self.device)
+        if not self.captured and meta.host_cu_q is not None and meta.max_q >= self.SSM_CHUNKED_MIN_ROWS:
+            count, packed, scratch = self._scan_chunks(meta, self._ops.distie_ssm_scan_chunk_rows(), H, N, P)
+            key = ("ssm_totals", count, H)
+            totals = meta.scratch.get(key)
+            if totals is None:
+                totals = meta.scratch[key] = torch.empty((count, H), dtype=torch.float32, device=self.device)
+            _check(self._ops.distie_ssm_scan_chunked(
+                x_ptr, _code(xbc), ld, d_ptr, ldd, dt_bias.data_ptr(), a_log.data_ptr(), skip.data_ptr(),
+                state.data_ptr(), out.data_ptr(), scratch.data_ptr(), totals.data_ptr(), packed.data_ptr(),
+                packed.data_ptr() + 16 * count, meta.state_slots.data_ptr(), count, meta.num_requests, H, P, N, G,
+                self._stream()), "ssm_scan_chunked")
+            _mark_written(state)
+            return out
+        if N > self._ops.distie_ssm_scan_max_state():
+            raise KernelError(f"ssm_scan: a state of {N} rows a head is beyond the row-by-row kernel")
+        _check(self._ops.distie_ssm_scan(x_ptr, _code(xbc), ld, d_ptr, ldd, dt_bias.data_ptr(), a_log.data_ptr(),
+                                         skip.data_ptr(), state.data_ptr(), out.data_ptr(), meta.cu_q.data_ptr(),
+                                         meta.state_slots.data_ptr(), meta.num_requests, H, P, N, G, self._stream()),
+               "ssm_scan")
+        _mark_written(state)
+        return out
+
+    def latent_norm_rope_write(self, down, q_rank, q_weight, kv_rank, kv_weight, eps, rot_dim, inv_freq, magnitude,
+                               neighbours, meta, group, k_cache, v_cache, write, out_dtype):
+        down = self.dense(down)
+        self._own(down, q_weight, kv_weight, k_cache, v_cache, inv_freq)
+        T, W = down.shape
+        if down.dtype != torch.float32 or W < q_rank + kv_rank + rot_dim or T != meta.num_tokens:
+            raise KernelError("latent_norm_rope_write: the down-projection is float32 [T, q_rank + kv_rank + rot_dim]")
+        for weight, size in ((q_weight, q_rank), (kv_weight, kv_rank)):
+            if size and (weight is None or weight.dtype != torch.float32 or tuple(weight.shape) != (size,)):
+                raise KernelError("latent_norm_rope_write: the norms' weights are float32 [rank]")
+        padded = k_cache.shape[-1]
+        if write:
+            self._check_cache(k_cache, v_cache, 1, meta.block_size, padded)
+            if k_cache.dtype != v_cache.dtype or padded < kv_rank + rot_dim:
+                raise KernelError("latent_norm_rope_write: one key/value head of at least kv_rank + rot_dim, in one dtype")
+        pairs = 0 if inv_freq is None else inv_freq.shape[0]
+        if pairs and 2 * pairs != rot_dim:
+            raise KernelError("latent_norm_rope_write: the rotation turns all of the rotated part")
+        table = self._rope_table(meta, inv_freq) if pairs else None
+        latent = torch.empty((T, q_rank), dtype=out_dtype, device=self.device) if q_rank else None
+        ptr = lambda t: t.data_ptr() if t is not None else None
+        _check(self._ops.distie_latent_norm_rope_write(
+            down.data_ptr(), W, q_rank, ptr(q_weight), kv_rank, kv_weight.data_ptr(), float(eps), rot_dim, ptr(table),
+            float(magnitude), 1 if neighbours else 0, ptr(latent), _CODES[out_dtype], k_cache.data_ptr(),
+            v_cache.data_ptr(), _code(k_cache), meta.groups[group].slots.data_ptr(), T, meta.block_size, padded,
+            1 if write else 0, self._stream()), "latent_norm_rope_write")
+        return latent
+
+    def heads_linear(self, x, weight, in_stride, out_stride, out=None):
+        x = self.dense(x)
+        self._own(x, weight, out)
+        if weight.dim() != 3:
+            raise KernelError("heads_linear: the weight is [heads, N, K]")
+        H, N, K = weight.shape
+        T = x.shape[0]
+        if x.shape[1] != H * in_stride or K > in_stride or N > out_stride:
+            raise KernelError("heads_linear: x is [T, heads * in_stride] with in_stride >= K, out_stride >= N")
+        if out is None:
+            make = torch.empty if N == out_stride else torch.zeros
+            out = make((T, H * out_stride), dtype=x.dtype, device=self.device)
+        elif out.dtype != x.dtype or tuple(out.shape) != (T, H * out_stride):
+            raise KernelError("heads_linear: out is [T, heads * out_stride] of x's dtype")
+        _check(self._ops.distie_heads_linear(x.data_ptr(), _code(x), in_stride, weight.data_ptr(), _code(weight),
+                                             out.data_ptr(), out_stride, T, H, N, K, self._stream()), "heads_linear")
+        return out
+
+    def rope_heads(self, x, in_stride, in_offset, out, out_stride, out_offset, num_heads, inv_freq, magnitude,
+                   neighbours, meta):
+        x = self.dense(x)
+        self._own(x, out, inv_freq)
+        T = x.shape[0]
+        if x.dtype != out.dtype or x.shape[1] != num_heads * in_stride or tuple(out.shape) != (T, num_heads * out_stride) \
+                or T != meta.num_tokens:
+            raise KernelError("rope_heads: x [T, heads * in_stride] and out [T, heads * out_stride] of one dtype")
+        table = self._rope_table(meta, inv_freq)
+        _check(self._ops.distie_rope_heads(x.data_ptr(), _code(x), in_stride, in_offset, out.data_ptr(), out_stride,
+                                           out_offset, T, num_heads, inv_freq.shape[0], table.data_ptr(),
+                                           float(magnitude), 1 if neighbours else 0, self._stream()), "rope_heads")
+        return out
+
+    def glu_mul(self, gate_up, kind):
+        if kind == "silu":
+            return self.silu_mul(gate_up)
+        if kind not in self.ACTIVATIONS:
+            raise KernelError(f"glu_mul: no activation named {kind!r}")
+        if isinstance(gate_up, (PendingNorm, PendingProduct)):
+            gate_up = self.dense(gate_up)
+        slices, source, dtype = 1, gate_up, gate_up.dtype
+        if isinstance(gate_up, PartialSums):
+            slices, source = gate_up.slices, gate_up.data
+        self._own(source)
+        rows, two = gate_up.shape
+        out = torch.empty((rows, two // 2), dtype=dtype, device=self.device)
+        _check(self._ops.distie_glu_mul(source.data_ptr(), _code(source), slices, out.data_ptr(), _code(out), rows,
+                                        two // 2, self.ACTIVATIONS[kind], self._stream()), "glu_mul")
         return out
 
     def silu_mul(self, gate_up):

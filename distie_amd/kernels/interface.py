@@ -107,8 +107,8 @@ class Ops(abc.ABC):
         table.view(-1)[index.long()] = value
 
     @abc.abstractmethod
-    def embed(self, ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
-        """ids int32 [T], table [V, C] -> float32 [T, C]."""
+    def embed(self, ids: torch.Tensor, table: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
+        """ids int32 [T], table [V, C] -> float32 [T, C], the rows times `scale` (in float32)."""
 
     @abc.abstractmethod
     def rmsnorm(self, x: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype) -> torch.Tensor:
@@ -213,12 +213,13 @@ class Ops(abc.ABC):
                                eps=eps, out_dtype=out_dtype)[1]
 
     def causal_conv(self, x: torch.Tensor, weight: torch.Tensor, state: Optional[torch.Tensor], meta: BatchMeta,
-                    residual: bool = False, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+                    residual: bool = False, bias: Optional[torch.Tensor] = None, act: Optional[str] = None) -> torch.Tensor:
         """x act [T, N] (or a view of columns with a row stride), weight [N, taps], bias float32 [N] or None
         -> y_t = bias + (x_t if residual) + sum_j weight[:, j] * x_(t - taps + 1 + j)
         within each request; what lies before the step's rows comes from `state` (float32 [slots + 1, taps - 1, N],
         the request's last taps - 1 inputs, oldest first, rows by `meta.state_slots`), which is moved on to the
-        end of the step's rows. Sums in float32, in the order of j."""
+        end of the step's rows. Sums in float32, in the order of j. `act`: one of `activation`'s names, applied to the
+        float32 sum before it is rounded (None: none)."""
         raise NotImplementedError(f"{type(self).__name__} has no convolution over time")
 
     def conv_rope_kv_write(self, product: torch.Tensor, conv_weight: Optional[torch.Tensor],
@@ -243,9 +244,10 @@ class Ops(abc.ABC):
         raise NotImplementedError(f"{type(self).__name__} has no convolution over time")
 
     def sigmoid_gate(self, x: torch.Tensor, num_heads: int, head_stride: int, width: int,
-                     gates: torch.Tensor) -> torch.Tensor:
+                     gates: torch.Tensor, per_head: bool = False) -> torch.Tensor:
         """x act [T, num_heads * head_stride], of which the first `width` of every head count; gates act
-        [T, num_heads * width] (or a view with a row stride) -> x * sigmoid(gates), act [T, num_heads * width]. `gates` None: the kept columns as they are."""
+        [T, num_heads * width] (or a view with a row stride) -> x * sigmoid(gates), act [T, num_heads * width]. `gates` None: the kept columns as they are.
+        `per_head`: gates act [T, num_heads] (or such a view), one number for all of a head's columns."""
         raise NotImplementedError(f"{type(self).__name__} has no gates")
 
     def decay_scan(self, product: torch.Tensor, state: torch.Tensor, decay: torch.Tensor, meta: BatchMeta,
@@ -258,12 +260,71 @@ class Ops(abc.ABC):
         raise NotImplementedError(f"{type(self).__name__} has no decayed state")
 
     def rmsnorm_gate(self, x: torch.Tensor, weight: torch.Tensor, eps: float, gates: Optional[torch.Tensor],
-                     out_dtype, group: Optional[int] = None, gate: str = "sigmoid") -> torch.Tensor:
+                     out_dtype, group: Optional[int] = None, gate: str = "sigmoid", gate_first: bool = False) -> torch.Tensor:
         """float32 [T, N] -> x / sqrt(mean(x^2) + eps) * weight * sigmoid(gates) in `out_dtype` (gates act [T, N]
         or a view with a row stride; None: no gate). `group`: the mean is taken over every run of `group` columns
         by itself (a head), and `weight` [group] is the same for all of them; None: over all N, weight [N].
-        `gate`: "sigmoid" or "silu" (times gates * sigmoid(gates))."""
+        `gate`: "sigmoid" or "silu" (times gates * sigmoid(gates)). With `group`, a weight of [N] is each column's own.
+        `gate_first`: the gate multiplies x in front of the norm, (x * gate) / sqrt(mean((x * gate)^2) + eps) * weight,
+        instead of its result."""
         raise NotImplementedError(f"{type(self).__name__} has no gated norm")
+
+    # ---- a state with one decay per head and token (state-space duality), attention over a shared latent
+    def ssm_scan(self, xbc: torch.Tensor, dt: torch.Tensor, dt_bias: torch.Tensor, a_log: torch.Tensor,
+                 skip: torch.Tensor, state: torch.Tensor, meta: BatchMeta, num_heads: int, value_dim: int,
+                 state_size: int, groups: int) -> torch.Tensor:
+        """The selective state-space recurrence in its scalar-decay form, over each request's rows in order. `xbc` act
+        [T, H * P + 2 * G * N] (or a view of columns): x (H heads of P = value_dim), then B and C (G groups of N =
+        state_size each; head h reads group h // (H / G)). `dt` act [T, H] (or a view), `dt_bias`, `a_log`, `skip`
+        float32 [H]. With d = softplus(dt + dt_bias) and a = exp(-exp(a_log) * d), per head
+
+            S <- a * S + d * B x^T   (S is N x P),        y = S^T C + skip * x.
+
+        `state` float32 [slots + 1, H, N, P] (rows by `meta.state_slots`) is read and left as the step's last row
+        leaves it. -> float32 [T, H * P]. Softplus, exponentials, the state, its products and sums in float32."""
+        raise NotImplementedError(f"{type(self).__name__} has no state-space recurrence")
+
+    def latent_norm_rope_write(self, down: torch.Tensor, q_rank: int, q_weight: Optional[torch.Tensor], kv_rank: int,
+                               kv_weight: torch.Tensor, eps: float, rot_dim: int, inv_freq: Optional[torch.Tensor],
+                               magnitude: float, neighbours: bool, meta: BatchMeta, group: int, k_cache: torch.Tensor,
+                               v_cache: torch.Tensor, write: bool, out_dtype) -> Optional[torch.Tensor]:
+        """Behind latent attention's stacked down-projection. `down` float32 [T, q_rank + kv_rank + rot_dim]: the
+        queries' latent, the keys' and values' latent, and one rotated key part for all heads. Both latents go through
+        an RMS norm of their own (x / sqrt(mean(x^2) + eps) * weight, float32). The normed queries' latent is returned
+        in `out_dtype` [T, q_rank] (None if q_rank is 0). If `write`, the token's slot of the cache gets the normed
+        latent c and the rotated key part as one key of one head, k_cache [pages, 1, P, DP] = (c, rotated part, zeros),
+        and c again as its value, v_cache [pages, 1, DP, P]. The key part's 2 * len(inv_freq) dimensions are turned by
+        the token's position, cosine and sine both times `magnitude`; `neighbours`: dimension 2i pairs with 2i + 1,
+        else i with i + len(inv_freq)."""
+        raise NotImplementedError(f"{type(self).__name__} has no latent attention")
+
+    def heads_linear(self, x: torch.Tensor, weight: torch.Tensor, in_stride: int, out_stride: int,
+                     out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """A product of its own for every head: x act [T, H * in_stride], head h's input its first K columns there;
+        weight [H, N, K] -> act [T, H * out_stride], head h's N results the first of its out_stride columns. The
+        other columns are zero, or what `out` (act [T, H * out_stride]) held. Sums in float32."""
+        raise NotImplementedError(f"{type(self).__name__} has no products by head")
+
+    def rope_heads(self, x: torch.Tensor, in_stride: int, in_offset: int, out: torch.Tensor, out_stride: int,
+                   out_offset: int, num_heads: int, inv_freq: torch.Tensor, magnitude: float, neighbours: bool,
+                   meta: BatchMeta) -> torch.Tensor:
+        """The 2 * len(inv_freq) columns at `in_offset` of every head of x (act [T, H * in_stride]), turned by the
+        token's position as in `latent_norm_rope_write`, written to the columns at `out_offset` of every head of `out`
+        (act [T, H * out_stride]) -> out."""
+        raise NotImplementedError(f"{type(self).__name__} has no rotation of head columns")
+
+    def latent_queries(self, q: torch.Tensor, key_up: torch.Tensor, num_heads: int, dim: int, rot_dim: int,
+                       padded_dim: int, inv_freq: Optional[torch.Tensor], magnitude: float, neighbours: bool,
+                       meta: BatchMeta) -> torch.Tensor:
+        """Latent attention's queries as the cache's one key head reads them. q act [T, H * (dim + rot_dim)], every
+        head (dim unrotated, rot_dim rotated); key_up [H, kv_rank, dim], head h's key expansion transposed. Since
+        q_h . (U_h c) = (U_h^T q_h) . c, head h's query against the cached (c, rotated key part) is
+        (key_up[h] q_h[:dim], turned q_h[dim:], zeros) -> act [T, H * padded_dim]. An implementation may fuse the two."""
+        out = self.heads_linear(q, key_up, dim + rot_dim, padded_dim)
+        if inv_freq is None:
+            raise NotImplementedError("latent attention's rotated part needs a rotation")
+        return self.rope_heads(q, dim + rot_dim, dim, out, padded_dim, key_up.shape[1], num_heads, inv_freq, magnitude,
+                               neighbours, meta)
 
     # ---- sums of normed sub-layer outputs, states with a decay of their own for every channel and token, routed
     # ---- feed-forwards. As above: an implementation that serves no model with them may leave them out.
@@ -373,6 +434,19 @@ class Ops(abc.ABC):
     def linear_act(self, x, weight: torch.Tensor, kind: str) -> torch.Tensor:
         """activation(linear(x, weight), kind); an implementation may fuse the two."""
         return self.activation(self.linear(x, weight), kind)
+
+    def glu_mul(self, gate_up, kind: str) -> torch.Tensor:
+        """[T, 2I] (or what `linear` returned) -> act(first half) * second half, [T, I]; `kind` one of `activation`'s
+        names. "silu" is `silu_mul`."""
+        if kind == "silu":
+            return self.silu_mul(gate_up)
+        raise NotImplementedError(f"{type(self).__name__} has no gated activation {kind!r}")
+
+    def linear_glu(self, x: torch.Tensor, gate_up_weight: torch.Tensor, kind: str) -> torch.Tensor:
+        """glu_mul(linear(x, gate_up_weight), kind); an implementation may fuse the two."""
+        if kind == "silu":
+            return self.linear_silu_mul(x, gate_up_weight)
+        return self.glu_mul(self.linear(x, gate_up_weight), kind)
 
     @abc.abstractmethod
     def silu_mul(self, gate_up: torch.Tensor) -> torch.Tensor:

@@ -6,7 +6,9 @@
 * a rotation of only the first dimensions of a head, with scaled frequencies (whatever the `position` part gives:
   its frequencies and the factor on cosine and sine);
 * keys of size `head_dim` and values of another size `value_dim`;
-* an output gate: the concatenated heads times sigmoid(W_g h), h being the mixer's input, before the output projection;
+* an output gate: the concatenated heads times sigmoid(W_g h), h being the mixer's input, before the output projection
+  (`output_gate` True: a gate for every value column, `g` [heads * value_dim, C]; "head": one number for each head,
+  `g` [heads, C]);
 * biases on q, k and v (`bias`: tensors `<q|k|v>.b`, added in the projection);
 * a query temperature by position (`q_temp` = {coef, every}): q at position p is multiplied by
   1 + coef * ln(floor((p + 1) / every) + 1), in float32, so that later queries weigh their keys more sharply;
@@ -60,7 +62,9 @@ class ConvGatedAttention(Mixer):
         self.window = p.get("window")
         self.keep = p.get("keep", self.window)          # how far back the cache must reach (None: everything)
         self.scale = float(p.get("scale", self.head_dim ** -0.5))
-        self.output_gate = bool(p.get("output_gate", True))
+        gate = p.get("output_gate", True)
+        self.output_gate = bool(gate)
+        self.gate_per_head = gate == "head"
         self.kv_from = p.get("kv_from")
         self.bias = bool(p.get("bias", False))
         temp = p.get("q_temp")
@@ -78,7 +82,8 @@ class ConvGatedAttention(Mixer):
         self.has_kv = self.kv_from is None
         q, k, v = self.num_heads * self.head_dim, self.num_kv_heads * self.head_dim, self.num_kv_heads * self.value_dim
         self.conv_channels = q + (k + v if self.has_kv else 0)
-        self.gate_width = self.num_heads * self.value_dim
+        self.out_width = self.num_heads * self.value_dim
+        self.gate_width = self.num_heads if self.gate_per_head else self.out_width
         self.in_weight = self.in_bias = self.conv_weight = self.out_weight = None
 
     def _projections(self):
@@ -111,7 +116,7 @@ class ConvGatedAttention(Mixer):
             specs["sink"] = ParamSpec((self.num_heads,))
         if self.output_gate:
             specs["g"] = ParamSpec((self.gate_width, self.hidden_size))
-        specs["o"] = ParamSpec((self.hidden_size, self.gate_width))
+        specs["o"] = ParamSpec((self.hidden_size, self.out_width))
         return specs
 
     def load(self, tensors) -> None:
@@ -157,7 +162,10 @@ class ConvGatedAttention(Mixer):
                                     self.padded_dim, self.scale, self.window, self.extras)
         if self.output_gate:
             gates = product[:, self.conv_channels:self.conv_channels + self.gate_width]
-            mixed = ops.sigmoid_gate(mixed, self.num_heads, self.padded_dim, self.value_dim, gates)
+            if self.gate_per_head:
+                mixed = ops.sigmoid_gate(mixed, self.num_heads, self.padded_dim, self.value_dim, gates, per_head=True)
+            else:
+                mixed = ops.sigmoid_gate(mixed, self.num_heads, self.padded_dim, self.value_dim, gates)
         elif self.padded_dim != self.value_dim:
             mixed = ops.sigmoid_gate(mixed, self.num_heads, self.padded_dim, self.value_dim, None)
         return ops.linear(mixed, self.out_weight)

@@ -10,7 +10,7 @@ from .base import Embedding, Head, ParamSpec, build_part, register_part
 
 class TokenEmbedding(Embedding):
     """`norm` (a norm's PartSpec, with its own prefix): the looked-up rows go through it before they become the
-    residual stream, which stays float32."""
+    residual stream, which stays float32. `scale`: what the looked-up rows are multiplied by, in float32."""
 
     def __init__(self, spec) -> None:
         super().__init__(spec)
@@ -18,6 +18,7 @@ class TokenEmbedding(Embedding):
         self.hidden_size = int(spec.params["hidden_size"])
         self.weight_name = spec.params.get("weight_name", "weight")      # the tensor's name behind the prefix
         self.norm = build_part("norm", spec.params["norm"]) if spec.params.get("norm") is not None else None
+        self.scale = float(spec.params.get("scale", 1.0))
         self.weight = None
 
     def parts(self):
@@ -32,7 +33,7 @@ class TokenEmbedding(Embedding):
         self.weight = tensors[self.weight_name].contiguous()
 
     def forward(self, ops, ids, meta):
-        hidden = ops.embed(ids, self.weight)
+        hidden = ops.embed(ids, self.weight) if self.scale == 1.0 else ops.embed(ids, self.weight, self.scale)
         return hidden if self.norm is None else ops.dense(self.norm.apply(ops, hidden, hidden.dtype))
 
 

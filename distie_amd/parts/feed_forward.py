@@ -10,8 +10,8 @@ from .base import FeedForward, ParamSpec, register_part
 
 
 class SwiGLU(FeedForward):
-    """down(silu(gate x) * up x); the tensors' names behind the prefix come from the spec (`gate_name`, `up_name`,
-    `down_name`)."""
+    """down(act(gate x) * up x), act = silu unless `activation` names another ("gelu_tanh"); the tensors' names
+    behind the prefix come from the spec (`gate_name`, `up_name`, `down_name`)."""
 
     def __init__(self, spec) -> None:
         super().__init__(spec)
@@ -20,6 +20,9 @@ class SwiGLU(FeedForward):
         self.gate_name = spec.params.get("gate_name", "gate_proj.weight")
         self.up_name = spec.params.get("up_name", "up_proj.weight")
         self.down_name = spec.params.get("down_name", "down_proj.weight")
+        self.activation = str(spec.params.get("activation", "silu"))
+        if self.activation not in ("silu", "gelu_tanh", "relu", "relu2"):
+            raise ValueError(f"no gated activation named {self.activation!r}")
         self.gate_up_weight = self.down_weight = None
 
     def param_specs(self):
@@ -36,11 +39,13 @@ class SwiGLU(FeedForward):
         self.down_weight = tensors[self.down_name].contiguous()
 
     def prepare(self, ops) -> None:
-        ops.prepare_linear(self.gate_up_weight, gated=True, role="gate_up")
+        ops.prepare_linear(self.gate_up_weight, gated=True if self.activation == "silu" else self.activation, role="gate_up")
         ops.prepare_linear(self.down_weight, role="down")
 
     def forward(self, ops, x, ctx):
-        return ops.linear(ops.linear_silu_mul(x, self.gate_up_weight), self.down_weight)
+        if self.activation == "silu":
+            return ops.linear(ops.linear_silu_mul(x, self.gate_up_weight), self.down_weight)
+        return ops.linear(ops.linear_glu(x, self.gate_up_weight, self.activation), self.down_weight)
 
 
 class DenseMLP(FeedForward):

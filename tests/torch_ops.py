@@ -17,8 +17,9 @@ class TorchOps(Ops):
     def __init__(self, device="cpu") -> None:
         self.device = torch.device(device)
 
-    def embed(self, ids, table):
-        return table[ids.long()].float()
+    def embed(self, ids, table, scale=1.0):
+        rows = table[ids.long()].float()
+        return rows if scale == 1.0 else rows * scale
 
     def rmsnorm(self, x, weight, eps, out_dtype):
         x = x.float()
@@ -140,9 +141,10 @@ class TorchOps(Ops):
             out += x.float()
         return out
 
-    def causal_conv(self, x, weight, state, meta, residual=False, bias=None):
+    def causal_conv(self, x, weight, state, meta, residual=False, bias=None, act=None):
         y = self._conv(x, weight, state, meta, residual)
-        return (y if bias is None else y + bias.float()).to(x.dtype)
+        y = y if bias is None else y + bias.float()
+        return (y if act is None else self.activation(y, act)).to(x.dtype)
 
     def conv_rope_kv_write(self, product, conv_weight, state, meta, group, k_cache, v_cache, inv_freq, magnitude,
                            num_heads, num_kv_heads, dim, value_dim, padded_dim, has_kv, write, q_temp=None, qk_norm=None):
@@ -182,10 +184,13 @@ class TorchOps(Ops):
             v_cache[slots // P, :, :value_dim, slots % P] = v.to(v_cache.dtype)
         return q.view(T, num_heads * padded_dim).to(product.dtype)
 
-    def sigmoid_gate(self, x, num_heads, head_stride, width, gates):
+    def sigmoid_gate(self, x, num_heads, head_stride, width, gates, per_head=False):
         T = x.shape[0]
-        kept = x.view(T, num_heads, head_stride)[..., :width].reshape(T, num_heads * width).float()
-        return (kept if gates is None else kept * torch.sigmoid(gates.float())).to(x.dtype)
+        kept = x.view(T, num_heads, head_stride)[..., :width].float()
+        if gates is not None:
+            g = torch.sigmoid(gates.float())
+            kept = kept * (g[:, :, None] if per_head else g.view(T, num_heads, width))
+        return kept.reshape(T, num_heads * width).to(x.dtype)
 
     def decay_scan(self, product, state, decay, meta, num_heads, dim, value_dim):
         T = product.shape[0]
@@ -204,14 +209,93 @@ class TorchOps(Ops):
             state[slots[b]] = s
         return out.view(T, num_heads * value_dim)
 
-    def rmsnorm_gate(self, x, weight, eps, gates, out_dtype, group=None, gate="sigmoid"):
+    def rmsnorm_gate(self, x, weight, eps, gates, out_dtype, group=None, gate="sigmoid", gate_first=False):
         T, N = x.shape
-        v = x.view(T, N // group, group) if group else x
-        y = (v / torch.sqrt((v ** 2).mean(-1, keepdim=True) + eps) * weight.float()).reshape(T, N)
+        factor = None
         if gates is not None:
             g = gates.float()
-            y = y * (torch.sigmoid(g) if gate == "sigmoid" else g * torch.sigmoid(g))
+            factor = torch.sigmoid(g) if gate == "sigmoid" else g * torch.sigmoid(g)
+        if gate_first and factor is not None:
+            x = x * factor
+        v = x.view(T, N // group, group) if group else x
+        w = weight.float()
+        if group and w.shape[0] == N:
+            w = w.view(N // group, group)
+        y = (v / torch.sqrt((v ** 2).mean(-1, keepdim=True) + eps) * w).reshape(T, N)
+        if factor is not None and not gate_first:
+            y = y * factor
         return y.to(out_dtype)
+
+    # ---- a state with one decay a head and token, attention over a shared latent
+    def ssm_scan(self, xbc, dt, dt_bias, a_log, skip, state, meta, num_heads, value_dim, state_size, groups):
+        T = xbc.shape[0]
+        H, P, N, G = num_heads, value_dim, state_size, groups
+        x = xbc[:, :H * P].float().view(T, H, P)
+        B = xbc[:, H * P:H * P + G * N].float().view(T, G, N).repeat_interleave(H // G, dim=1)
+        C = xbc[:, H * P + G * N:H * P + 2 * G * N].float().view(T, G, N).repeat_interleave(H // G, dim=1)
+        d = torch.nn.functional.softplus(dt.float() + dt_bias.float(), threshold=80.0)
+        a = torch.exp(-torch.exp(a_log.float()) * d)
+        out = torch.zeros(T, H, P, dtype=torch.float32, device=xbc.device)
+        cu, slots = meta.cu_q.tolist(), meta.state_slots.tolist()
+        for b in range(meta.num_requests):
+            s = state[slots[b]]
+            for t in range(cu[b], cu[b + 1]):
+                s = a[t][:, None, None] * s + d[t][:, None, None] * B[t][:, :, None] * x[t][:, None, :]
+                out[t] = torch.einsum("hnp,hn->hp", s, C[t]) + skip.float()[:, None] * x[t]
+            state[slots[b]] = s
+        return out.view(T, H * P)
+
+    @staticmethod
+    def _turn(x, positions, inv_freq, magnitude, neighbours):
+        """x [..., 2 * pairs] with rows by token -> turned by each token's position."""
+        pairs = inv_freq.shape[0]
+        ang = positions.float()[:, None] * inv_freq.float()[None, :]
+        shape = [x.shape[0]] + [1] * (x.dim() - 2) + [pairs]
+        cos, sin = (ang.cos() * magnitude).view(shape), (ang.sin() * magnitude).view(shape)
+        if neighbours:
+            a, b = x[..., 0::2], x[..., 1::2]
+            return torch.stack([a * cos - b * sin, b * cos + a * sin], -1).flatten(-2)
+        a, b = x[..., :pairs], x[..., pairs:]
+        return torch.cat([a * cos - b * sin, b * cos + a * sin], -1)
+
+    def latent_norm_rope_write(self, down, q_rank, q_weight, kv_rank, kv_weight, eps, rot_dim, inv_freq, magnitude,
+                               neighbours, meta, group, k_cache, v_cache, write, out_dtype):
+        down = down.float()
+        latent = self._rms(down[:, :q_rank], q_weight, eps).to(out_dtype) if q_rank else None
+        if write:
+            c = self._rms(down[:, q_rank:q_rank + kv_rank], kv_weight, eps)
+            r = down[:, q_rank + kv_rank:q_rank + kv_rank + rot_dim]
+            if inv_freq is not None:
+                r = self._turn(r, meta.positions, inv_freq, magnitude, neighbours)
+            P = k_cache.shape[2]
+            slots = meta.groups[group].slots.long()
+            k_cache[slots // P, 0, slots % P, :kv_rank] = c.to(k_cache.dtype)
+            k_cache[slots // P, 0, slots % P, kv_rank:kv_rank + rot_dim] = r.to(k_cache.dtype)
+            v_cache[slots // P, 0, :kv_rank, slots % P] = c.to(v_cache.dtype)
+        return latent
+
+    def heads_linear(self, x, weight, in_stride, out_stride, out=None):
+        T = x.shape[0]
+        H, N, K = weight.shape
+        if out is None:
+            out = torch.zeros(T, H * out_stride, dtype=x.dtype, device=x.device)
+        y = torch.einsum("thk,hnk->thn", x.view(T, H, in_stride)[..., :K].float(), weight.float())
+        out.view(T, H, out_stride)[..., :N] = y.to(x.dtype)
+        return out
+
+    def rope_heads(self, x, in_stride, in_offset, out, out_stride, out_offset, num_heads, inv_freq, magnitude,
+                   neighbours, meta):
+        T = x.shape[0]
+        n = 2 * inv_freq.shape[0]
+        part = x.view(T, num_heads, in_stride)[..., in_offset:in_offset + n].float()
+        out.view(T, num_heads, out_stride)[..., out_offset:out_offset + n] = \
+            self._turn(part, meta.positions, inv_freq, magnitude, neighbours).to(out.dtype)
+        return out
+
+    def glu_mul(self, gate_up, kind):
+        inter = gate_up.shape[1] // 2
+        g, u = gate_up[:, :inter].float(), gate_up[:, inter:].float()
+        return (self.activation(g, kind) * u).to(gate_up.dtype)
 
     # ---- sums of normed terms, states with their own decays, routers
     @staticmethod
