@@ -17,7 +17,7 @@ serves it), points at batch 1 and 32, and a cache that takes the card's memory u
 the time to the first token and the time per output token after it, defined as the reference's load
 generator defines them (benchmarks/load/stats.py:29-34, 67-86).
 
-`--design musutar|duparax|sekazen [--size w1024|w2048|w4096]`: prefill and decode of that decoder beside a Qwen2
+`--design musutar|duparax|sekazen|dufelix [--size w1024|w2048|w4096]`: prefill and decode of that decoder beside a Qwen2
 decoder of equal width, depth, heads and weights, at layer sizes of real models; one JSON line with both for every size.
 
 Random weights N(0, 0.02), seeded uniform token ids.
@@ -278,6 +278,32 @@ def sekazen_config(size):
             "logit_softcap": 50.0, "layers": layers}
 
 
+def dufelix_config(size):
+    """Groups of four layers: two of latent attention (a latent of 192 and a rotated key part of 64 for all heads,
+    queries through a latent of three eighths of the width, a sink for each head), a state-space layer (heads of 64
+    channels on twice the width, a state of 128 rows, four taps) and one of grouped-query attention with half of every
+    head turned and a gate for each head; norms on both sides of every sub-layer, gelu-gated dense feed-forwards."""
+    z = DESIGN_SIZES[size]
+    stretch = {"factor": 8.0, "original": 1024, "fast": 32.0, "slow": 1.0}
+    layers = []
+    for i in range(z["layers"]):
+        mlp = {"kind": "dense", "ff": z["ff"]}
+        if i % 4 < 2:
+            mixer = {"heads": z["heads"], "dim": z["dim"], "rot_dim": 64, "vdim": z["dim"], "kv_rank": 192,
+                     "q_rank": 3 * z["width"] // 8, "scale": (z["dim"] + 64) ** -0.5,
+                     "rot": {"base": 10000.0, "dims": 64, "scaling": stretch}}
+            layers.append({"type": "latent_attention", "mixer": mixer, "mlp": mlp})
+        elif i % 4 == 2:
+            mixer = {"heads": 2 * z["width"] // 64, "vdim": 64, "state": 128, "groups": 1, "conv": 4, "norm_groups": 1}
+            layers.append({"type": "mamba2", "mixer": mixer, "mlp": mlp})
+        else:
+            mixer = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["dim"],
+                     "scale": z["dim"] ** -0.5, "rot": {"base": 10000.0, "dims": z["dim"] // 2, "scaling": stretch}}
+            layers.append({"type": "attention", "mixer": mixer, "mlp": mlp})
+    return {"architecture": "Dufelix", "vocab": DESIGN_VOCAB, "width": z["width"], "norm": {"eps": 1e-6},
+            "embedding": {"scale": 8.0}, "layers": layers}
+
+
 def qwen2_of_weights(size, layer_weights):
     """The Qwen2 decoder with the same width, depth and heads and a feed-forward sized so that its layers hold as many
     weights as the other design's layers do on average."""
@@ -296,7 +322,7 @@ def design_pair(design, size):
     from distie_amd.config import config_from_dict
     from distie_amd.engine.model import Model
 
-    config = sekazen_config(size) if design == "sekazen" else duparax_config(size)
+    config = {"sekazen": sekazen_config, "duparax": duparax_config, "dufelix": dufelix_config}[design](size)
     total = 0
     for name, spec in Model.declare(config_from_dict(config).model_spec()).items():
         if name.startswith("l"):
@@ -368,7 +394,7 @@ def main() -> int:
                         help="size the cache from free memory (the default for --shape 32b and --serve: 0.9)")
     parser.add_argument("--packed-weights", default=None, metavar="ROLES",
                         help="packed copies only for these products (qkv,attn_out,gate_up,down,head); 'none' for no copies")
-    parser.add_argument("--design", default=None, choices=["musutar", "duparax", "sekazen"],
+    parser.add_argument("--design", default=None, choices=["musutar", "duparax", "sekazen", "dufelix"],
                         help="instead of the workload above: this design beside a Qwen2 decoder of equal size, prefill and decode")
     parser.add_argument("--size", default=None, choices=sorted(DESIGN_SIZES), help="with --design: one size instead of all")
     args = parser.parse_args()

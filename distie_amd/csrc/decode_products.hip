@@ -355,7 +355,7 @@ __global__ __launch_bounds__(64 * WR * WK) void decode_product_kernel(ProductArg
       for (int i = 0; i < 4; ++i) {
         float gate = acc[i], u = up[i];
         if (p.bias != nullptr && n0 + i < half) { gate += p.bias[n0 + i]; u += p.bias[half + n0 + i]; }
-        v[i] = gate / (1.f + expf(-gate)) * u;
+        v[i] = gate_activation(gate, p.rotary.act) * u;
       }
       if (n0 + 3 < half && half % 4 == 0) {
         *reinterpret_cast<uint2*>(y + static_cast<int64_t>(r) * half + n0) = pack_bf16x4(v);
@@ -531,7 +531,9 @@ extern "C" int distie_decode_norm_product(const float* residual, const float* no
                                           void* v_cache, int heads, int kv_heads, int dim, int block_size, int write,
                                           hipStream_t stream) {
   if (M <= 0) return 0;
-  if (M > 16 || N <= 0 || K <= 0 || K % 8 != 0 || !norm_fits(K) || mode < 0 || mode > 2 ||
+  const int act = mode >> 8;            // gated: the activation on the gate, above the low eight bits
+  mode &= 0xff;
+  if (M > 16 || N <= 0 || K <= 0 || K % 8 != 0 || !norm_fits(K) || mode < 0 || mode > 2 || act < 0 || act > 4 ||
       residual == nullptr || norm_weight == nullptr)
     return DISTIE_BAD_ARGUMENT;
   ProductArgs p = {};
@@ -545,6 +547,7 @@ extern "C" int distie_decode_norm_product(const float* residual, const float* no
   if (mode == PK_GATED) {
     if (N % 2 != 0) return DISTIE_BAD_ARGUMENT;
     p.row_blocks = (N / 2 + 7) / 8;
+    p.rotary.act = act;
     // four row blocks share a workgroup's x, one wave each
     return launch_norm<PK_GATED, OUT_BF16, 4, 1, 16>(p, stream);
   }

@@ -13,22 +13,22 @@
 // ---------------------------------------------------------------- embedding
 template <typename W>
 __global__ void embed_kernel(const int32_t* __restrict__ ids, const W* __restrict__ table,
-                             float* __restrict__ out, int width, int vocab) {
+                             float* __restrict__ out, int width, int vocab, float scale) {
   const int64_t t = blockIdx.x;
   int64_t id = ids[t];
   if (id < 0 || id >= vocab) id = 0;  // ids are validated on the host; never read outside the table
   const W* row = table + id * width;
   float* dst = out + t * width;
-  for (int i = threadIdx.x; i < width; i += blockDim.x) dst[i] = to_float(row[i]);
+  for (int i = threadIdx.x; i < width; i += blockDim.x) dst[i] = to_float(row[i]) * scale;      // (times one is exact)
 }
 
 extern "C" int distie_embed(const int32_t* ids, const void* table, int table_dtype, float* out,
-                            int tokens, int width, int vocab, hipStream_t stream) {
+                            int tokens, int width, int vocab, float scale, hipStream_t stream) {
   if (tokens <= 0) return 0;
   if (width <= 0 || vocab <= 0) return DISTIE_BAD_ARGUMENT;
   const int threads = width >= 1024 ? 256 : 64;
   DISTIE_DISPATCH(table_dtype, W,
-                  embed_kernel<W><<<tokens, threads, 0, stream>>>(ids, static_cast<const W*>(table), out, width, vocab));
+                  embed_kernel<W><<<tokens, threads, 0, stream>>>(ids, static_cast<const W*>(table), out, width, vocab, scale));
   return launch_status();
 }
 

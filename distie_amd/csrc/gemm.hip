@@ -416,7 +416,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_packed_kernel(const bf16_t* _
         if (n >= half) continue;
         float gate = acc[i], u = up[i];
         if (bias != nullptr) { gate += bias[n]; u += bias[half + n]; }
-        y[static_cast<int64_t>(r) * half + n] = from_float<Y>(gate / (1.f + expf(-gate)) * u);
+        y[static_cast<int64_t>(r) * half + n] = from_float<Y>(gate_activation(gate, rotary.act) * u);
       }
     }
   } else if constexpr (MODE == PK_ROTARY) {
@@ -492,7 +492,9 @@ static int packed_waves(int K) {
 extern "C" int distie_gemm_packed_bf16(const void* x, const void* w_packed, const float* bias, void* y, int y_dtype,
                                        int M, int N, int K, int gated, hipStream_t stream) {
   if (M <= 0) return 0;
-  if (M > 256 || N <= 0 || K <= 0 || K % 8 != 0 || (gated && N % 2 != 0)) return DISTIE_BAD_ARGUMENT;
+  const int act = gated >> 8;           // the activation on the gate, above the low eight bits
+  gated &= 0xff;
+  if (M > 256 || N <= 0 || K <= 0 || K % 8 != 0 || (gated && N % 2 != 0) || act < 0 || act > 4) return DISTIE_BAD_ARGUMENT;
   int slices = 1, k_per_slice = (K + SK_KSTEP - 1) / SK_KSTEP * SK_KSTEP;
   if (!gated) skinny_plan(N, K, &slices, &k_per_slice);
   if (slices > 1 && y_dtype != DISTIE_F32) return DISTIE_BAD_ARGUMENT;
@@ -500,7 +502,8 @@ extern "C" int distie_gemm_packed_bf16(const void* x, const void* w_packed, cons
   dim3 grid(row_blocks, slices, (M + 15) / 16);
   const bf16_t* xb = static_cast<const bf16_t*>(x);
   const bf16_t* wb = static_cast<const bf16_t*>(w_packed);
-  const RotaryOut none = {};
+  RotaryOut none = {};
+  none.act = act;
   if (gated && M <= 8) {
     // The gated product is not cut along K (the activation needs the whole sum), so a row block's K goes to the four
     // waves of a workgroup, which add their sums through LDS: up to 8 rows of x that is faster than one wave a row
@@ -552,6 +555,7 @@ constexpr int WD_MAX_BLOCKS = 6;
 // sum over K, which this kernel cuts into slices, so it is left to the kernel that adds the slices.
 struct HeadRows {
   int heads, kv_heads, dim;
+  int act;                    // gated products only: the activation on the gate (gate_activation)
 };
 
 template <typename Y, int MODE, int MB, int WD_WAVES>
@@ -679,7 +683,7 @@ __global__ __launch_bounds__(64 * WD_WAVES) void gemm_packed_wide_kernel(const b
         for (int i = 0; i < 4; ++i) {
           float gate = acc[b][i], u = up[i];
           if (bias != nullptr && n0 + i < half) { gate += bias[n0 + i]; u += bias[half + n0 + i]; }
-          v[i] = gate / (1.f + expf(-gate)) * u;
+          v[i] = gate_activation(gate, head_rows.act) * u;
         }
 #pragma unroll
         for (int i = 0; i < 4; ++i)
@@ -731,7 +735,7 @@ extern "C" int distie_gemm_packed_wide_slices(int N, int K) {
 // Up to 256 rows of x, at most 96 a pass. mode 0: y [M, N] of y_dtype, or float32 [slices, M, N] when the plan cuts K
 // (distie_gemm_packed_wide_slices); 1 (gated): [M, N / 2].
 static int packed_wide_launch(const bf16_t* x, const bf16_t* w, const float* bias, void* y, int y_dtype, int M, int N,
-                              int K, int mode, int pass_blocks, hipStream_t stream, HeadRows head_rows = HeadRows{0, 0, 0}) {
+                              int K, int mode, int pass_blocks, hipStream_t stream, HeadRows head_rows = HeadRows{0, 0, 0, 0}) {
   const int row_blocks = mode == PK_GATED ? (N / 2 + 7) / 8 : (N + 15) / 16;
   int slices = 1, tiles_per_slice = 4 * ((K + SK_KSTEP - 1) / SK_KSTEP);
   if (mode != PK_GATED) wide_plan(row_blocks, K, &slices, &tiles_per_slice);
@@ -782,9 +786,11 @@ extern "C" int distie_gemm_packed_wide_bf16(const void* x, const void* w_packed,
                                             int y_dtype, int M, int N, int K, int gated, int pass_blocks,
                                             hipStream_t stream) {
   if (M <= 0) return 0;
-  if (M > 256 || N <= 0 || K <= 0 || K % 8 != 0 || (gated && N % 2 != 0)) return DISTIE_BAD_ARGUMENT;
+  const int act = gated >> 8;           // the activation on the gate, above the low eight bits
+  gated &= 0xff;
+  if (M > 256 || N <= 0 || K <= 0 || K % 8 != 0 || (gated && N % 2 != 0) || act < 0 || act > 4) return DISTIE_BAD_ARGUMENT;
   return packed_wide_launch(static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w_packed), bias, y, y_dtype, M, N,
-                            K, gated ? PK_GATED : PK_PLAIN, pass_blocks, stream);
+                            K, gated ? PK_GATED : PK_PLAIN, pass_blocks, stream, HeadRows{0, 0, 0, act});
 }
 
 // The stacked q/k/v product alone, on the ROTARY copy of its weight, for 17 rows of x and more against a weight large

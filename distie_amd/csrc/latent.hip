@@ -171,6 +171,70 @@ heads_linear_rows_kernel(const X* __restrict__ x, int lx, const W* __restrict__ 
   }
 }
 
+// The same product on the matrix cores, bfloat16 operands and float32 sums (v_mfma_f32_32x32x16_bf16): a wave owns 32
+// rows of x by 32 * NB rows of a head's weight and walks k sixteen at a time; both operands are rows with k innermost,
+// so a lane's eight values are one 16-byte load (row = lane % 32, k = 8 * (lane / 32) ..). The weights of a head are
+// small (they stay in the caches), so nothing goes through LDS. A workgroup is WT x WN waves; blockIdx = (tile of n,
+// tile of t, head). K and the row strides are multiples of 8.
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 hl_bf16x8;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float hl_floatx16;
+
+template <int WT, int WN, int NB>
+__global__ void __launch_bounds__(64 * WT * WN)
+heads_linear_mfma_kernel(const bf16_t* __restrict__ x, int lx, const bf16_t* __restrict__ w, bf16_t* __restrict__ out,
+                         int lo, int T, int H, int N, int K) {
+  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+  const int h = blockIdx.z;
+  const int t0 = (blockIdx.y * WT + wave / WN) * 32;
+  const int n0 = (blockIdx.x * WN + wave % WN) * 32 * NB;
+  if (t0 >= T || n0 >= N) return;
+  const int r = lane % 32, kk = 8 * (lane / 32);
+  const bool t_in = t0 + r < T;
+  const bf16_t* xr = x + (static_cast<int64_t>(t_in ? t0 + r : t0) * H + h) * lx + kk;
+  const bf16_t* wr[NB];
+  bool n_in[NB];
+#pragma unroll
+  for (int b = 0; b < NB; ++b) {
+    n_in[b] = n0 + 32 * b + r < N;
+    wr[b] = w + (static_cast<int64_t>(h) * N + (n_in[b] ? n0 + 32 * b + r : n0)) * K + kk;
+  }
+  hl_floatx16 acc[NB];
+#pragma unroll
+  for (int b = 0; b < NB; ++b)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[b][i] = 0.f;
+  for (int k0 = 0; k0 < K; k0 += 32) {
+    // two k-steps' loads under way together
+    hl_bf16x8 a[2], bw[2][NB];
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      const int k = k0 + 16 * s;
+      const bool k_in = k + kk < K;
+      a[s] = (t_in && k_in) ? *reinterpret_cast<const hl_bf16x8*>(xr + k) : hl_bf16x8{};
+#pragma unroll
+      for (int b = 0; b < NB; ++b)
+        bw[s][b] = (n_in[b] && k_in) ? *reinterpret_cast<const hl_bf16x8*>(wr[b] + k) : hl_bf16x8{};
+    }
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+      for (int b = 0; b < NB; ++b) acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[s], bw[s][b], acc[b], 0, 0, 0);
+  }
+  // acc[b][4 i + j]: row t0 + 8 i + 4 (lane / 32) + j of x, weight row n0 + 32 b + lane % 32
+#pragma unroll
+  for (int b = 0; b < NB; ++b) {
+    const int n = n0 + 32 * b + r;
+    if (n >= N) continue;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int t = t0 + 8 * i + 4 * (lane / 32) + j;
+        if (t < T) out[(static_cast<int64_t>(t) * H + h) * lo + n] = static_cast<bf16_t>(acc[b][4 * i + j]);
+      }
+  }
+}
+
 // ---------------------------------------------------------------------------------------------------
 // out[t, h * E + e] = x[t, h * ldh + e] * sigmoid(gates[t * ldg + h]): one gate a head
 template <typename X, typename G, typename O>
@@ -225,6 +289,20 @@ extern "C" int distie_heads_linear(const void* x, int dtype, int lx, const void*
                                    int H, int N, int K, hipStream_t stream) {
   if (T <= 0) return 0;
   if (H < 1 || N < 1 || K < 1 || lx < K || lo < N || H > 65535) return DISTIE_BAD_ARGUMENT;
+  if (dtype == DISTIE_BF16 && w_dtype == DISTIE_BF16 && K % 8 == 0 && lx % 8 == 0 &&
+      reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0) {
+    const bf16_t* xb = static_cast<const bf16_t*>(x);
+    const bf16_t* wb = static_cast<const bf16_t*>(w);
+    bf16_t* ob = static_cast<bf16_t*>(out);
+    if (T <= 32) {
+      heads_linear_mfma_kernel<1, 4, 1><<<dim3((N + 127) / 128, 1, H), 256, 0, stream>>>(xb, lx, wb, ob, lo, T, H, N, K);
+    } else {
+      const dim3 grid((N + 127) / 128, (T + 63) / 64, H);
+      if (grid.y > 65535) return DISTIE_BAD_ARGUMENT;
+      heads_linear_mfma_kernel<2, 2, 2><<<grid, 256, 0, stream>>>(xb, lx, wb, ob, lo, T, H, N, K);
+    }
+    return launch_status();
+  }
   if (T <= 2 * HLR_ROWS) {
     const int64_t items = static_cast<int64_t>(H) * N;
     const dim3 grid(static_cast<unsigned>((items + 3) / 4), (T + HLR_ROWS - 1) / HLR_ROWS);

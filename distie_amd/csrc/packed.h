@@ -18,7 +18,18 @@ struct RotaryOut {
   bf16_t* k_cache;            // [pages, kv_heads, block_size, D]
   bf16_t* v_cache;            // [pages, kv_heads, D, block_size]
   int heads, kv_heads, dim, block_size, write;
+  int act;                    // gated products only: the activation on the gate (see gate_activation)
 };
+
+// The activation on the gate of a gated product: 0 silu; else 1 + the kind as `distie_activation` numbers them
+// (1: the square of max(z, 0), 3: the tanh form of gelu, 4: max(z, 0)). The C interface takes it in the bits above
+// the low eight of its `gated` / `mode` argument.
+static __device__ __forceinline__ float gate_activation(float z, int act) {
+  if (act == 0 || act == 2) return z / (1.f + expf(-z));
+  if (act == 3) return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+  const float p = fmaxf(z, 0.f);
+  return act == 1 ? p * p : p;
+}
 
 static __device__ __forceinline__ uint2 pack_bf16x4(const float v[4]) {
   uint32_t h[4];

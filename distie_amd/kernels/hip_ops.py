@@ -283,7 +283,7 @@ class HipOps(Ops):
     def _declare(self) -> None:
         o = self._ops
         o.distie_scatter_i32.argtypes = [_P, _P, _P, _I, _L, _P]
-        o.distie_embed.argtypes = [_P, _P, _I, _P, _I, _I, _I, _P]
+        o.distie_embed.argtypes = [_P, _P, _I, _P, _I, _I, _I, _F, _P]
         o.distie_rmsnorm.argtypes = [_P, _P, _I, _I, _P, _I, _P, _I, _I, _I, _F, _P]
         o.distie_rope_kv_write.argtypes = [_P, _I, _I, _P, _I, _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P]
         o.distie_rope_table.argtypes = [_P, _P, _P, _I, _I, _P]
@@ -410,9 +410,7 @@ class HipOps(Ops):
         self._own(ids, table)
         out = torch.empty((ids.shape[0], table.shape[1]), dtype=torch.float32, device=self.device)
         _check(self._ops.distie_embed(ids.data_ptr(), table.data_ptr(), _code(table), out.data_ptr(),
-                                      ids.shape[0], table.shape[1], table.shape[0], self._stream()), "embed")
-        if scale != 1.0 and out.numel():
-            _check(self._ops.distie_scale_f32(out.data_ptr(), out.numel(), float(scale), self._stream()), "scale_f32")
+                                      ids.shape[0], table.shape[1], table.shape[0], float(scale), self._stream()), "embed")
         return out
 
     def _norm_later(self, residual, weight, out_dtype) -> bool:
@@ -579,16 +577,24 @@ class HipOps(Ops):
         return out
 
     def linear_silu_mul(self, x, gate_up_weight):
+        return self.linear_glu(x, gate_up_weight, "silu")
+
+    def linear_glu(self, x, gate_up_weight, kind):
+        """The gated product with the activation in its epilogue, on the GATED copy of the weight (steps of few rows);
+        else the product, then `glu_mul`."""
+        if kind not in self.ACTIVATIONS:
+            raise KernelError(f"linear_glu: no activation named {kind!r}")
+        gated = 1 if kind == "silu" else 1 | ((self.ACTIVATIONS[kind] + 1) << 8)
         packed = getattr(gate_up_weight, "_distie_gated", None)
         if isinstance(x, PendingNorm) and packed is not None and gate_up_weight.shape[1] == x.shape[1]:
             N, K = gate_up_weight.shape
             if packed.numel() != self._packed_elements(N, K, True):
                 raise KernelError("linear_silu_mul: the packed copy does not belong to this weight")
             out = torch.empty((x.shape[0], N // 2), dtype=torch.bfloat16, device=self.device)
-            return self._norm_product(x, packed, None, out, 1, N)
+            return self._norm_product(x, packed, None, out, gated, N)
         x = self.dense(x)
         if packed is None or x.dtype != torch.bfloat16 or x.shape[0] > self._packed_rows(x.shape[0], *gate_up_weight.shape):
-            return self.silu_mul(self.linear(x, gate_up_weight))
+            return self.glu_mul(self.linear(x, gate_up_weight), kind)
         self._own(x)
         M, K = x.shape
         N = gate_up_weight.shape[0]
@@ -599,10 +605,10 @@ class HipOps(Ops):
         out = torch.empty((M, N // 2), dtype=x.dtype, device=self.device)
         if M <= self.ONE_WAVE_MAX_ROWS:
             _check(self._ops.distie_gemm_packed_bf16(x.data_ptr(), packed.data_ptr(), None, out.data_ptr(), _code(out),
-                                                     M, N, K, 1, self._stream()), "gemm_packed_bf16")
+                                                     M, N, K, gated, self._stream()), "gemm_packed_bf16")
         else:
             _check(self._ops.distie_gemm_packed_wide_bf16(
-                x.data_ptr(), packed.data_ptr(), None, out.data_ptr(), _code(out), M, N, K, 1,
+                x.data_ptr(), packed.data_ptr(), None, out.data_ptr(), _code(out), M, N, K, gated,
                 self._pass_blocks(M, N * K), self._stream()), "gemm_packed_wide_bf16")
         return out
 

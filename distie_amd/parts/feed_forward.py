@@ -39,7 +39,7 @@ class SwiGLU(FeedForward):
         self.down_weight = tensors[self.down_name].contiguous()
 
     def prepare(self, ops) -> None:
-        ops.prepare_linear(self.gate_up_weight, gated=True if self.activation == "silu" else self.activation, role="gate_up")
+        ops.prepare_linear(self.gate_up_weight, gated=True, role="gate_up")
         ops.prepare_linear(self.down_weight, role="down")
 
     def forward(self, ops, x, ctx):
