@@ -22,16 +22,21 @@ __device__ __forceinline__ float sigmoidf(float x) { return 1.f / (1.f + __expf(
 // table [T, pairs] holds (cos, sin) of every pair's angle; both are multiplied by `magnitude`. `neighbours`: the pair
 // is (2 j, 2 j + 1), else (j, j + pairs). What lies beyond kv_rank + rot_dim in a key and beyond kv_rank in a value
 // was zero when the cache was made and is never written.
+// `down` may be `slices` partial sums of the product, `slice_stride` elements apart (added in order while the row is
+// read into LDS, where both norms and the rotation find it).
 template <typename O, typename C>
-__global__ void latent_norm_rope_write_kernel(const float* __restrict__ down, int64_t ld, int q_rank,
-                                              const float* __restrict__ q_weight, int kv_rank,
+__global__ void latent_norm_rope_write_kernel(const float* __restrict__ down, int slices, int64_t slice_stride, int64_t ld,
+                                              int q_rank, const float* __restrict__ q_weight, int kv_rank,
                                               const float* __restrict__ kv_weight, float eps, int rot_dim,
                                               const float2* __restrict__ table, float magnitude, int neighbours,
                                               O* __restrict__ latent, C* __restrict__ k_cache, C* __restrict__ v_cache,
                                               const int32_t* __restrict__ slots, int P, int DP, int write) {
+  extern __shared__ float row[];               // q_rank + kv_rank + rot_dim values
   __shared__ float scratch[16];
   const int64_t t = blockIdx.x;
-  const float* row = down + t * ld;
+  const int width = q_rank + kv_rank + rot_dim;
+  for (int c = threadIdx.x; c < width; c += blockDim.x) row[c] = sum_strided(down + t * ld + c, slices, slice_stride);
+  __syncthreads();
   if (q_rank > 0) {
     float sq = 0.f;
     for (int c = threadIdx.x; c < q_rank; c += blockDim.x) sq += row[c] * row[c];
@@ -179,59 +184,116 @@ heads_linear_rows_kernel(const X* __restrict__ x, int lx, const W* __restrict__ 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 hl_bf16x8;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float hl_floatx16;
 
-template <int WT, int WN, int NB>
+// What a fused call adds behind a head's product, for latent attention's queries: the 2 * pairs columns at `offset_in`
+// of the head's input, turned by the token's angle, go to the columns behind the product's N results, and the rest of
+// the head's `lo` output columns is zeroed. pairs 0: nothing of this.
+struct QueryTail {
+  const float2* table;        // [T, pairs] cosine and sine
+  float magnitude;
+  int pairs, offset_in, neighbours;
+};
+
+// SLICED: x is float32 [slices, T, H * lx], partial sums of the product that made it, added in order and rounded to
+// bfloat16 once (what a kernel that adds them up in front of this one would hand over).
+template <bool SLICED>
+__device__ __forceinline__ float load_x(const void* x, int64_t at, int slices, int64_t slice_stride) {
+  if constexpr (SLICED) return sum_strided(static_cast<const float*>(x) + at, slices, slice_stride);
+  else return to_float(static_cast<const bf16_t*>(x)[at]);
+}
+
+template <int WT, int WN, int NB, bool SLICED>
 __global__ void __launch_bounds__(64 * WT * WN)
-heads_linear_mfma_kernel(const bf16_t* __restrict__ x, int lx, const bf16_t* __restrict__ w, bf16_t* __restrict__ out,
-                         int lo, int T, int H, int N, int K) {
+heads_linear_mfma_kernel(const void* __restrict__ x, int slices, int64_t slice_stride, int lx, const bf16_t* __restrict__ w,
+                         bf16_t* __restrict__ out, int lo, int T, int H, int N, int K, QueryTail tail) {
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
   const int h = blockIdx.z;
   const int t0 = (blockIdx.y * WT + wave / WN) * 32;
   const int n0 = (blockIdx.x * WN + wave % WN) * 32 * NB;
-  if (t0 >= T || n0 >= N) return;
-  const int r = lane % 32, kk = 8 * (lane / 32);
-  const bool t_in = t0 + r < T;
-  const bf16_t* xr = x + (static_cast<int64_t>(t_in ? t0 + r : t0) * H + h) * lx + kk;
-  const bf16_t* wr[NB];
-  bool n_in[NB];
+  if (t0 < T && n0 < N) {
+    const int r = lane % 32, kk = 8 * (lane / 32);
+    const bool t_in = t0 + r < T;
+    const int64_t x_at = (static_cast<int64_t>(t_in ? t0 + r : t0) * H + h) * lx + kk;
+    const bf16_t* wr[NB];
+    bool n_in[NB];
 #pragma unroll
-  for (int b = 0; b < NB; ++b) {
-    n_in[b] = n0 + 32 * b + r < N;
-    wr[b] = w + (static_cast<int64_t>(h) * N + (n_in[b] ? n0 + 32 * b + r : n0)) * K + kk;
-  }
-  hl_floatx16 acc[NB];
-#pragma unroll
-  for (int b = 0; b < NB; ++b)
-#pragma unroll
-    for (int i = 0; i < 16; ++i) acc[b][i] = 0.f;
-  for (int k0 = 0; k0 < K; k0 += 32) {
-    // two k-steps' loads under way together
-    hl_bf16x8 a[2], bw[2][NB];
-#pragma unroll
-    for (int s = 0; s < 2; ++s) {
-      const int k = k0 + 16 * s;
-      const bool k_in = k + kk < K;
-      a[s] = (t_in && k_in) ? *reinterpret_cast<const hl_bf16x8*>(xr + k) : hl_bf16x8{};
-#pragma unroll
-      for (int b = 0; b < NB; ++b)
-        bw[s][b] = (n_in[b] && k_in) ? *reinterpret_cast<const hl_bf16x8*>(wr[b] + k) : hl_bf16x8{};
+    for (int b = 0; b < NB; ++b) {
+      n_in[b] = n0 + 32 * b + r < N;
+      wr[b] = w + (static_cast<int64_t>(h) * N + (n_in[b] ? n0 + 32 * b + r : n0)) * K + kk;
     }
+    hl_floatx16 acc[NB];
 #pragma unroll
-    for (int s = 0; s < 2; ++s)
+    for (int b = 0; b < NB; ++b)
 #pragma unroll
-      for (int b = 0; b < NB; ++b) acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[s], bw[s][b], acc[b], 0, 0, 0);
-  }
-  // acc[b][4 i + j]: row t0 + 8 i + 4 (lane / 32) + j of x, weight row n0 + 32 b + lane % 32
+      for (int i = 0; i < 16; ++i) acc[b][i] = 0.f;
+    for (int k0 = 0; k0 < K; k0 += 32) {
+      // two k-steps' loads under way together
+      hl_bf16x8 a[2], bw[2][NB];
 #pragma unroll
-  for (int b = 0; b < NB; ++b) {
-    const int n = n0 + 32 * b + r;
-    if (n >= N) continue;
+      for (int s = 0; s < 2; ++s) {
+        const int k = k0 + 16 * s;
+        const bool k_in = k + kk < K;
+        a[s] = hl_bf16x8{};
+        if (t_in && k_in) {
+          if constexpr (SLICED) {
+            const float* xf = static_cast<const float*>(x) + x_at + k;
+            float4 lo4 = *reinterpret_cast<const float4*>(xf), hi4 = *reinterpret_cast<const float4*>(xf + 4);
+            for (int q = 1; q < slices; ++q) {
+              const float4 l2 = *reinterpret_cast<const float4*>(xf + q * slice_stride);
+              const float4 h2 = *reinterpret_cast<const float4*>(xf + q * slice_stride + 4);
+              lo4.x += l2.x, lo4.y += l2.y, lo4.z += l2.z, lo4.w += l2.w;
+              hi4.x += h2.x, hi4.y += h2.y, hi4.z += h2.z, hi4.w += h2.w;
+            }
+            a[s][0] = static_cast<bf16_t>(lo4.x), a[s][1] = static_cast<bf16_t>(lo4.y);
+            a[s][2] = static_cast<bf16_t>(lo4.z), a[s][3] = static_cast<bf16_t>(lo4.w);
+            a[s][4] = static_cast<bf16_t>(hi4.x), a[s][5] = static_cast<bf16_t>(hi4.y);
+            a[s][6] = static_cast<bf16_t>(hi4.z), a[s][7] = static_cast<bf16_t>(hi4.w);
+          } else {
+            a[s] = *reinterpret_cast<const hl_bf16x8*>(static_cast<const bf16_t*>(x) + x_at + k);
+          }
+        }
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int t = t0 + 8 * i + 4 * (lane / 32) + j;
-        if (t < T) out[(static_cast<int64_t>(t) * H + h) * lo + n] = static_cast<bf16_t>(acc[b][4 * i + j]);
+        for (int b = 0; b < NB; ++b)
+          bw[s][b] = (n_in[b] && k_in) ? *reinterpret_cast<const hl_bf16x8*>(wr[b] + k) : hl_bf16x8{};
       }
+#pragma unroll
+      for (int s = 0; s < 2; ++s)
+#pragma unroll
+        for (int b = 0; b < NB; ++b) acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[s], bw[s][b], acc[b], 0, 0, 0);
+    }
+    // acc[b][4 i + j]: row t0 + 8 i + 4 (lane / 32) + j of x, weight row n0 + 32 b + lane % 32
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+      const int n = n0 + 32 * b + r;
+      if (n >= N) continue;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int t = t0 + 8 * i + 4 * (lane / 32) + j;
+          if (t < T) out[(static_cast<int64_t>(t) * H + h) * lo + n] = static_cast<bf16_t>(acc[b][4 * i + j]);
+        }
+    }
+  }
+  if (tail.pairs == 0 || blockIdx.x != 0) return;
+  // the workgroup's rows of x, this head: the turned part behind the product's columns, zeros behind that
+  const int first = blockIdx.y * WT * 32;
+  const int rows = min(WT * 32, T - first);
+  for (int i = threadIdx.x; i < rows * tail.pairs; i += blockDim.x) {
+    const int t = first + i / tail.pairs, j = i % tail.pairs;
+    const int a = tail.neighbours ? 2 * j : j, b = tail.neighbours ? 2 * j + 1 : j + tail.pairs;
+    const float2 cs = tail.table[static_cast<int64_t>(t) * tail.pairs + j];
+    const int64_t in = (static_cast<int64_t>(t) * H + h) * lx + tail.offset_in;
+    // (the unfused path rounds the summed product before it is turned)
+    const float u = to_float(static_cast<bf16_t>(load_x<SLICED>(x, in + a, slices, slice_stride)));
+    const float v = to_float(static_cast<bf16_t>(load_x<SLICED>(x, in + b, slices, slice_stride)));
+    bf16_t* to = out + (static_cast<int64_t>(t) * H + h) * lo + N;
+    to[a] = static_cast<bf16_t>(u * cs.x * tail.magnitude - v * cs.y * tail.magnitude);
+    to[b] = static_cast<bf16_t>(v * cs.x * tail.magnitude + u * cs.y * tail.magnitude);
+  }
+  const int pad = lo - N - 2 * tail.pairs;
+  for (int i = threadIdx.x; i < rows * pad; i += blockDim.x) {
+    const int t = first + i / pad;
+    out[(static_cast<int64_t>(t) * H + h) * lo + N + 2 * tail.pairs + i % pad] = static_cast<bf16_t>(0.f);
   }
 }
 
@@ -250,21 +312,25 @@ __global__ void head_gate_kernel(const X* __restrict__ x, int ldh, int E, const 
 
 }  // namespace
 
-extern "C" int distie_latent_norm_rope_write(const float* down, int64_t ld, int q_rank, const float* q_weight, int kv_rank,
+// the widest row (q_rank + kv_rank + rot_dim) that the kernel stages
+extern "C" int distie_latent_norm_max_width() { return 12288; }
+
+extern "C" int distie_latent_norm_rope_write(const float* down, int slices, int64_t ld, int q_rank, const float* q_weight, int kv_rank,
                                              const float* kv_weight, float eps, int rot_dim, const void* table,
                                              float magnitude, int neighbours, void* latent, int out_dtype, void* k_cache,
                                              void* v_cache, int cache_dtype, const int32_t* slots, int T, int P, int DP,
                                              int write, hipStream_t stream) {
   if (T <= 0) return 0;
   if (q_rank < 0 || kv_rank < 1 || rot_dim < 0 || rot_dim % 2 || ld < static_cast<int64_t>(q_rank) + kv_rank + rot_dim ||
+      slices < 1 || q_rank + kv_rank + rot_dim > 12288 ||
       (q_rank > 0 && (q_weight == nullptr || latent == nullptr)) || kv_weight == nullptr ||
       (write && (k_cache == nullptr || v_cache == nullptr || slots == nullptr || P < 1 || DP < kv_rank + rot_dim)))
     return DISTIE_BAD_ARGUMENT;
   const int widest = q_rank > kv_rank ? q_rank : kv_rank;
   const int threads = widest >= 256 ? 256 : (widest >= 128 ? 128 : 64);
   DISTIE_DISPATCH(out_dtype, O, DISTIE_DISPATCH(cache_dtype, C,
-      latent_norm_rope_write_kernel<O, C><<<T, threads, 0, stream>>>(
-          down, ld, q_rank, q_weight, kv_rank, kv_weight, eps, rot_dim, static_cast<const float2*>(table), magnitude,
+      latent_norm_rope_write_kernel<O, C><<<T, threads, sizeof(float) * (q_rank + kv_rank + rot_dim), stream>>>(
+          down, slices, static_cast<int64_t>(T) * ld, ld, q_rank, q_weight, kv_rank, kv_weight, eps, rot_dim, static_cast<const float2*>(table), magnitude,
           neighbours, static_cast<O*>(latent), static_cast<C*>(k_cache), static_cast<C*>(v_cache), slots, P, DP, write)));
   return launch_status();
 }
@@ -285,24 +351,52 @@ extern "C" int distie_rope_heads(const void* x, int dtype, int lx, int offset_in
 // the most rows of x that the kernel for few rows is chosen for
 extern "C" int distie_heads_linear_few_rows() { return 2 * HLR_ROWS; }
 
+static bool heads_linear_mfma_fits(const void* x, int dtype, const void* w, int w_dtype, int lx, int K, int slices) {
+  const bool x_ok = slices > 1 ? (dtype == DISTIE_F32 && lx % 4 == 0) : (dtype == DISTIE_BF16 && lx % 8 == 0);
+  return x_ok && w_dtype == DISTIE_BF16 && K % 8 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 &&
+         reinterpret_cast<uintptr_t>(w) % 16 == 0;
+}
+
+// x: bfloat16 [T, H * lx], or (slices > 1) float32 [slices, T, H * lx]
+static int heads_linear_mfma(const void* x, int slices, int lx, const void* w, void* out, int lo, int T, int H, int N, int K,
+                             QueryTail tail, hipStream_t stream) {
+  const bf16_t* wb = static_cast<const bf16_t*>(w);
+  bf16_t* ob = static_cast<bf16_t*>(out);
+  const int64_t stride = static_cast<int64_t>(T) * H * lx;
+  if (T <= 32) {
+    const dim3 grid((N + 127) / 128, 1, H);
+    if (slices > 1) heads_linear_mfma_kernel<1, 4, 1, true><<<grid, 256, 0, stream>>>(x, slices, stride, lx, wb, ob, lo, T, H, N, K, tail);
+    else heads_linear_mfma_kernel<1, 4, 1, false><<<grid, 256, 0, stream>>>(x, 1, 0, lx, wb, ob, lo, T, H, N, K, tail);
+  } else {
+    const dim3 grid((N + 127) / 128, (T + 63) / 64, H);
+    if (grid.y > 65535) return DISTIE_BAD_ARGUMENT;
+    if (slices > 1) heads_linear_mfma_kernel<2, 2, 2, true><<<grid, 256, 0, stream>>>(x, slices, stride, lx, wb, ob, lo, T, H, N, K, tail);
+    else heads_linear_mfma_kernel<2, 2, 2, false><<<grid, 256, 0, stream>>>(x, 1, 0, lx, wb, ob, lo, T, H, N, K, tail);
+  }
+  return launch_status();
+}
+
+// Latent attention's queries in one launch, bfloat16 on the matrix cores: head h's first K input columns times
+// w[h] ([N, K]) into the first N of its `lo` output columns, the next 2 * pairs input columns turned by the token's
+// angle into the columns behind them, zeros in the rest. x: bfloat16 [T, H * lx] or float32 [slices, T, H * lx].
+// Returns DISTIE_BAD_ARGUMENT for what the kernel does not take (the caller then composes the unfused operations).
+extern "C" int distie_latent_queries(const void* x, int dtype, int slices, int lx, const void* w, int w_dtype, void* out,
+                                     int lo, int T, int H, int N, int K, int pairs, const void* table, float magnitude,
+                                     int neighbours, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (H < 1 || N < 1 || K < 1 || pairs < 1 || slices < 1 || H > 65535 || lx < K + 2 * pairs || lo < N + 2 * pairs ||
+      table == nullptr || !heads_linear_mfma_fits(x, dtype, w, w_dtype, lx, K, slices) || (slices == 1 && dtype != DISTIE_BF16))
+    return DISTIE_BAD_ARGUMENT;
+  return heads_linear_mfma(x, slices, lx, w, out, lo, T, H, N, K,
+                           QueryTail{static_cast<const float2*>(table), magnitude, pairs, K, neighbours}, stream);
+}
+
 extern "C" int distie_heads_linear(const void* x, int dtype, int lx, const void* w, int w_dtype, void* out, int lo, int T,
                                    int H, int N, int K, hipStream_t stream) {
   if (T <= 0) return 0;
   if (H < 1 || N < 1 || K < 1 || lx < K || lo < N || H > 65535) return DISTIE_BAD_ARGUMENT;
-  if (dtype == DISTIE_BF16 && w_dtype == DISTIE_BF16 && K % 8 == 0 && lx % 8 == 0 &&
-      reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0) {
-    const bf16_t* xb = static_cast<const bf16_t*>(x);
-    const bf16_t* wb = static_cast<const bf16_t*>(w);
-    bf16_t* ob = static_cast<bf16_t*>(out);
-    if (T <= 32) {
-      heads_linear_mfma_kernel<1, 4, 1><<<dim3((N + 127) / 128, 1, H), 256, 0, stream>>>(xb, lx, wb, ob, lo, T, H, N, K);
-    } else {
-      const dim3 grid((N + 127) / 128, (T + 63) / 64, H);
-      if (grid.y > 65535) return DISTIE_BAD_ARGUMENT;
-      heads_linear_mfma_kernel<2, 2, 2><<<grid, 256, 0, stream>>>(xb, lx, wb, ob, lo, T, H, N, K);
-    }
-    return launch_status();
-  }
+  if (heads_linear_mfma_fits(x, dtype, w, w_dtype, lx, K, 1))
+    return heads_linear_mfma(x, 1, lx, w, out, lo, T, H, N, K, QueryTail{nullptr, 1.f, 0, 0, 0}, stream);
   if (T <= 2 * HLR_ROWS) {
     const int64_t items = static_cast<int64_t>(H) * N;
     const dim3 grid(static_cast<unsigned>((items + 3) / 4), (T + HLR_ROWS - 1) / HLR_ROWS);

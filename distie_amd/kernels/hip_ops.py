@@ -326,8 +326,9 @@ class HipOps(Ops):
         o.distie_activation.argtypes = [_P, _I, _I, _P, _I, _L, _I, _P]
         o.distie_decay_scan.argtypes = [_P, _I, _L, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P]
         o.distie_decay_scan_chunked.argtypes = [_P, _I, _L, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]
-        o.distie_latent_norm_rope_write.argtypes = [_P, _L, _I, _P, _I, _P, _F, _I, _P, _F, _I, _P, _I, _P, _P, _I, _P,
+        o.distie_latent_norm_rope_write.argtypes = [_P, _I, _L, _I, _P, _I, _P, _F, _I, _P, _F, _I, _P, _I, _P, _P, _I, _P,
                                                     _I, _I, _I, _I, _P]
+        o.distie_latent_queries.argtypes = [_P, _I, _I, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P, _F, _I, _P]
         o.distie_rope_heads.argtypes = [_P, _I, _I, _I, _P, _I, _I, _I, _I, _I, _P, _F, _I, _P]
         o.distie_heads_linear.argtypes = [_P, _I, _I, _P, _I, _P, _I, _I, _I, _I, _I, _P]
         o.distie_head_gate.argtypes = [_P, _I, _I, _I, _P, _I, _L, _P, _I, _I, _I, _P]
@@ -878,7 +879,9 @@ class HipOps(Ops):
         """May return `PartialSums` (see there)."""
         return self._linear(x, weight, bias, x.dtype, partial_ok=True, lazy=True)
 
-    def linear_f32out(self, x, weight, bias=None, scale=1.0):
+    def linear_f32out(self, x, weight, bias=None, scale=1.0, partial=False):
+        if partial and scale == 1.0:
+            return self._linear(x, weight, bias, torch.float32, partial_ok=True)
         out = self._linear(x, weight, bias, torch.float32)
         if scale != 1.0:
             _check(self._ops.distie_scale_f32(out.data_ptr(), out.numel(), float(scale), self._stream()), "scale_f32")
@@ -1679,9 +1682,16 @@ class HipOps(Ops):
 
     def latent_norm_rope_write(self, down, q_rank, q_weight, kv_rank, kv_weight, eps, rot_dim, inv_freq, magnitude,
                                neighbours, meta, group, k_cache, v_cache, write, out_dtype):
-        down = self.dense(down)
+        slices = 1
+        if isinstance(down, PartialSums) and down.dtype == torch.float32 and \
+                down.shape[1] <= self._ops.distie_latent_norm_max_width():
+            slices, down = down.slices, down.data.view(-1, down.data.shape[-1])        # added up while they are read
+        else:
+            down = self.dense(down)
         self._own(down, q_weight, kv_weight, k_cache, v_cache, inv_freq)
-        T, W = down.shape
+        T, W = down.shape[0] // slices, down.shape[1]
+        if slices == 1 and W > self._ops.distie_latent_norm_max_width():
+            raise KernelError("latent_norm_rope_write: the down-projection is wider than the kernel's row")
         if down.dtype != torch.float32 or W < q_rank + kv_rank + rot_dim or T != meta.num_tokens:
             raise KernelError("latent_norm_rope_write: the down-projection is float32 [T, q_rank + kv_rank + rot_dim]")
         for weight, size in ((q_weight, q_rank), (kv_weight, kv_rank)):
@@ -1699,11 +1709,35 @@ class HipOps(Ops):
         latent = torch.empty((T, q_rank), dtype=out_dtype, device=self.device) if q_rank else None
         ptr = lambda t: t.data_ptr() if t is not None else None
         _check(self._ops.distie_latent_norm_rope_write(
-            down.data_ptr(), W, q_rank, ptr(q_weight), kv_rank, kv_weight.data_ptr(), float(eps), rot_dim, ptr(table),
+            down.data_ptr(), slices, W, q_rank, ptr(q_weight), kv_rank, kv_weight.data_ptr(), float(eps), rot_dim, ptr(table),
             float(magnitude), 1 if neighbours else 0, ptr(latent), _CODES[out_dtype], k_cache.data_ptr(),
             v_cache.data_ptr(), _code(k_cache), meta.groups[group].slots.data_ptr(), T, meta.block_size, padded,
             1 if write else 0, self._stream()), "latent_norm_rope_write")
         return latent
+
+    def latent_queries(self, q, key_up, num_heads, dim, rot_dim, padded_dim, inv_freq, magnitude, neighbours, meta):
+        """One launch on the matrix cores for bfloat16 steps (the product's partial sums added up while they are read);
+        else the product by head, then the rotation."""
+        kv_rank = key_up.shape[1]
+        slices, source, dtype = 1, q, getattr(q, "dtype", None)
+        if isinstance(q, PartialSums):
+            slices, source = q.slices, q.data
+        fused = dtype == torch.bfloat16 and key_up.dtype == torch.bfloat16 and inv_freq is not None and \
+            isinstance(source, torch.Tensor) and 2 * inv_freq.shape[0] == rot_dim and dim % 8 == 0 and \
+            (dim + rot_dim) % 8 == 0 and tuple(key_up.shape) == (num_heads, kv_rank, dim) and \
+            tuple(q.shape) == (meta.num_tokens, num_heads * (dim + rot_dim)) and padded_dim >= kv_rank + rot_dim
+        if not fused:
+            return super().latent_queries(self.dense(q), key_up, num_heads, dim, rot_dim, padded_dim, inv_freq, magnitude,
+                                          neighbours, meta)
+        self._own(source, key_up, inv_freq)
+        T = meta.num_tokens
+        table = self._rope_table(meta, inv_freq)
+        out = torch.empty((T, num_heads * padded_dim), dtype=torch.bfloat16, device=self.device)
+        _check(self._ops.distie_latent_queries(
+            source.data_ptr(), _code(source), slices, dim + rot_dim, key_up.data_ptr(), _code(key_up), out.data_ptr(),
+            padded_dim, T, num_heads, kv_rank, dim, rot_dim // 2, table.data_ptr(), float(magnitude),
+            1 if neighbours else 0, self._stream()), "latent_queries")
+        return out
 
     def heads_linear(self, x, weight, in_stride, out_stride, out=None):
         x = self.dense(x)

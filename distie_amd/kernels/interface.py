@@ -168,8 +168,10 @@ class Ops(abc.ABC):
 
     @abc.abstractmethod
     def linear_f32out(self, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
-                      scale: float = 1.0) -> torch.Tensor:
-        """As `linear`, result in float32 and not rounded (the logits; what enters a recurrence), times `scale`."""
+                      scale: float = 1.0, partial: bool = False) -> torch.Tensor:
+        """As `linear`, result in float32 and not rounded (the logits; what enters a recurrence), times `scale`.
+        `partial`: as with `linear`, the result may come in a form of the implementation's own, for the operations
+        that say they take it (`latent_norm_rope_write`) and for `dense`."""
 
     @abc.abstractmethod
     def rope_kv_write(self, qkv: torch.Tensor, meta: BatchMeta, group: int, k_cache: torch.Tensor,
@@ -288,7 +290,8 @@ class Ops(abc.ABC):
                                kv_weight: torch.Tensor, eps: float, rot_dim: int, inv_freq: Optional[torch.Tensor],
                                magnitude: float, neighbours: bool, meta: BatchMeta, group: int, k_cache: torch.Tensor,
                                v_cache: torch.Tensor, write: bool, out_dtype) -> Optional[torch.Tensor]:
-        """Behind latent attention's stacked down-projection. `down` float32 [T, q_rank + kv_rank + rot_dim]: the
+        """Behind latent attention's stacked down-projection. `down` float32 [T, q_rank + kv_rank + rot_dim] (or what
+        `linear_f32out(..., partial=True)` returned): the
         queries' latent, the keys' and values' latent, and one rotated key part for all heads. Both latents go through
         an RMS norm of their own (x / sqrt(mean(x^2) + eps) * weight, float32). The normed queries' latent is returned
         in `out_dtype` [T, q_rank] (None if q_rank is 0). If `write`, the token's slot of the cache gets the normed
@@ -316,10 +319,12 @@ class Ops(abc.ABC):
     def latent_queries(self, q: torch.Tensor, key_up: torch.Tensor, num_heads: int, dim: int, rot_dim: int,
                        padded_dim: int, inv_freq: Optional[torch.Tensor], magnitude: float, neighbours: bool,
                        meta: BatchMeta) -> torch.Tensor:
-        """Latent attention's queries as the cache's one key head reads them. q act [T, H * (dim + rot_dim)], every
+        """Latent attention's queries as the cache's one key head reads them. q act [T, H * (dim + rot_dim)] (or what
+        `linear` returned), every
         head (dim unrotated, rot_dim rotated); key_up [H, kv_rank, dim], head h's key expansion transposed. Since
         q_h . (U_h c) = (U_h^T q_h) . c, head h's query against the cached (c, rotated key part) is
         (key_up[h] q_h[:dim], turned q_h[dim:], zeros) -> act [T, H * padded_dim]. An implementation may fuse the two."""
+        q = self.dense(q)
         out = self.heads_linear(q, key_up, dim + rot_dim, padded_dim)
         if inv_freq is None:
             raise NotImplementedError("latent attention's rotated part needs a rotation")

@@ -112,12 +112,11 @@ class LatentAttention(Mixer):
     def forward(self, ops, x, ctx, cache, writes_cache: bool):
         k_cache, v_cache = cache["k"], cache["v"]
         inv_freq, magnitude = self.position.rotary(), self.position.rotary_magnitude()
-        down = ops.linear_f32out(x, self.down_weight)
+        down = ops.linear_f32out(x, self.down_weight, partial=True)
         latent = ops.latent_norm_rope_write(down, self.q_rank, self.q_norm, self.kv_rank, self.kv_norm, self.eps,
                                             self.rot_dim, inv_freq, magnitude, self.neighbours, ctx.meta, cache.group,
                                             k_cache, v_cache, writes_cache, ctx.act_dtype)
-        q = ops.dense(ops.linear(latent, self.q_up))
-        q = ops.latent_queries(q, self.key_up, self.num_heads, self.head_dim, self.rot_dim, self.padded_dim, inv_freq,
+        q = ops.latent_queries(ops.linear(latent, self.q_up), self.key_up, self.num_heads, self.head_dim, self.rot_dim, self.padded_dim, inv_freq,
                                magnitude, self.neighbours, ctx.meta)
         mixed = ops.paged_attention(q, ctx.meta, cache.group, k_cache, v_cache, self.num_heads, 1, self.padded_dim,
                                     self.scale, None, self.extras)

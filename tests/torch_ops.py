@@ -36,7 +36,7 @@ class TorchOps(Ops):
             y = y + bias.float()
         return y.to(x.dtype)
 
-    def linear_f32out(self, x, weight, bias=None, scale=1.0):
+    def linear_f32out(self, x, weight, bias=None, scale=1.0, partial=False):
         y = x.float() @ weight.float().T
         if bias is not None:
             y = y + bias.float()
