@@ -592,6 +592,82 @@ __global__ void causal_conv_bf16x8_kernel(const bf16_t* __restrict__ x, int64_t 
   if (cu_q[b + 1] - first == 1 && taps > 1) shift_state8(own, taps, c0, N, self);
 }
 
+__device__ __forceinline__ void load_f32x8(const float* __restrict__ p, float v[8]);
+
+// The same for filters of TAPS = 2, 3 or 4 taps: the filters, the last TAPS - 1 inputs and the sums stay in registers
+// (every index is known when the kernel is compiled), and a thread walks R rows of the step one after the other, so a
+// row of x is read once and serves the TAPS rows that see it. Where a row is its request's first of the step, the
+// inputs before it come from the request's state.
+template <int TAPS, int R>
+__global__ void causal_conv_bf16_taps_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __restrict__ weight,
+                                             float* __restrict__ state, bf16_t* __restrict__ out, int64_t ldo, int mode,
+                                             const float* __restrict__ bias, const int32_t* __restrict__ cu_q,
+                                             const int32_t* __restrict__ token_request,
+                                             const int32_t* __restrict__ state_slots, int N, int T) {
+  const int c0 = 8 * (blockIdx.y * blockDim.x + threadIdx.x);
+  if (c0 >= N) return;
+  const int t0 = blockIdx.x * R;
+  float w[TAPS][8];                     // w[j][e]: tap j of channel c0 + e
+  {
+    float flat[8 * TAPS];
+#pragma unroll
+    for (int q = 0; q < TAPS; ++q) unpack_bf16x8(load16(weight + static_cast<int64_t>(c0) * TAPS + 8 * q), flat + 8 * q);
+#pragma unroll
+    for (int e = 0; e < 8; ++e)
+#pragma unroll
+      for (int j = 0; j < TAPS; ++j) w[j][e] = flat[e * TAPS + j];
+  }
+  float add[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) add[e] = bias != nullptr ? bias[c0 + e] : 0.f;
+  float win[TAPS - 1][8];               // the inputs of the TAPS - 1 rows before this one, oldest first
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int t = t0 + r;
+    if (t >= T) break;
+    const int b = token_request[t];
+    const int first = cu_q[b];
+    const int i = t - first;
+    float* own = state + static_cast<int64_t>(state_slots[b]) * (TAPS - 1) * N;
+    if (r == 0 || i == 0) {
+#pragma unroll
+      for (int k = 0; k < TAPS - 1; ++k) {
+        const int back = TAPS - 1 - k;
+        if (back <= i) unpack_bf16x8(load16(x + static_cast<int64_t>(t - back) * ldx + c0), win[k]);
+        else load_f32x8(own + static_cast<int64_t>(TAPS - 1 - (back - i)) * N + c0, win[k]);
+      }
+    }
+    float self[8], acc[8];
+    unpack_bf16x8(load16(x + static_cast<int64_t>(t) * ldx + c0), self);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      float sum = 0.f;
+#pragma unroll
+      for (int k = 0; k < TAPS - 1; ++k) sum += w[k][e] * win[k][e];
+      sum += w[TAPS - 1][e] * self[e];
+      if (mode & 1) sum += self[e];
+      sum += add[e];
+      acc[e] = (mode >> 1) ? activate(sum, (mode >> 1) - 1) : sum;
+    }
+    *reinterpret_cast<uint4*>(out + static_cast<int64_t>(t) * ldo + c0) = pack_bf16x8(acc);
+#pragma unroll
+    for (int k = 0; k + 1 < TAPS - 1; ++k)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) win[k][e] = win[k + 1][e];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) win[TAPS - 2][e] = self[e];
+    if (i == 0 && cu_q[b + 1] - first == 1) {
+      // a request that brings one row: the window, moved on by that row, is its new state
+#pragma unroll
+      for (int k = 0; k < TAPS - 1; ++k) {
+        float4* to = reinterpret_cast<float4*>(own + static_cast<int64_t>(k) * N + c0);
+        to[0] = float4{win[k][0], win[k][1], win[k][2], win[k][3]};
+        to[1] = float4{win[k][4], win[k][5], win[k][6], win[k][7]};
+      }
+    }
+  }
+}
+
 // conv_rope_kv_write for steps of 32 rows and more, bfloat16 products and caches, D, E and the number of pairs multiples of 8, DP == D or the
 // places beyond D zeroed by eight. Blocks 0 .. T-1: q and k of one token (a thread turns eight pairs, or copies eight
 // single dimensions). The blocks behind them: v for 16 tokens each; a thread owns one channel of v and, where
@@ -1236,6 +1312,23 @@ extern "C" int distie_causal_conv(const void* x, int x_dtype, int64_t ldx, const
       ldo % 8 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0 && reinterpret_cast<uintptr_t>(state) % 16 == 0) {
     const int items = N / 8;
     const int threads8 = items >= 256 ? 256 : (items >= 128 ? 128 : 64);
+    if (taps >= 2 && taps <= 4 && reinterpret_cast<uintptr_t>(weight) % 16 == 0) {
+      const bf16_t* xb = static_cast<const bf16_t*>(x);
+      const bf16_t* wb = static_cast<const bf16_t*>(weight);
+      bf16_t* ob = static_cast<bf16_t*>(out);
+      // few rows: a thread a row, narrow blocks, so that the chip has something to do; many: four rows a thread
+      const int rows = T >= 256 ? 4 : 1;
+      const int threads = T >= 256 ? threads8 : 64;
+      const dim3 grid((T + rows - 1) / rows, (items + threads - 1) / threads);
+#define DISTIE_CONV_TAPS(TAPS)                                                                                          \
+  if (rows == 4) causal_conv_bf16_taps_kernel<TAPS, 4><<<grid, threads, 0, stream>>>(                                   \
+      xb, ldx, wb, state, ob, ldo, residual, bias, cu_q, token_request, state_slots, N, T);                             \
+  else causal_conv_bf16_taps_kernel<TAPS, 1><<<grid, threads, 0, stream>>>(                                             \
+      xb, ldx, wb, state, ob, ldo, residual, bias, cu_q, token_request, state_slots, N, T)
+      if (taps == 2) { DISTIE_CONV_TAPS(2); } else if (taps == 3) { DISTIE_CONV_TAPS(3); } else { DISTIE_CONV_TAPS(4); }
+#undef DISTIE_CONV_TAPS
+      return launch_status();
+    }
     causal_conv_bf16x8_kernel<<<dim3(T, (items + threads8 - 1) / threads8), threads8, 0, stream>>>(
         static_cast<const bf16_t*>(x), ldx, static_cast<const bf16_t*>(weight), taps, state, static_cast<bf16_t*>(out), ldo,
         residual, bias, cu_q, token_request, state_slots, N);

@@ -94,6 +94,7 @@ ssm_scan_kernel(const X* __restrict__ xbc, int64_t ld, const X* __restrict__ dt,
 // of ln a inside the chunk (l_i <= 0, falling), S the state in front of the chunk:
 //   sums:     U[n][p]  = sum_j exp(l_L - l_j) d_j B_j[n] x_j[p],  total = exp(l_L)            (each chunk alone)
 //   states:   S_next   = total * S + U, chunk after chunk; S (the state in front) takes U's place in the scratch
+//   pairs:    (C_i . B_j) for the chunk's rows, once for every group of heads that shares B and C
 //   outputs:  y_i[p]   = exp(l_i) sum_n C_i[n] S[n][p] + sum_{j<=i} exp(l_i - l_j) d_j (C_i . B_j) x_j[p] + skip x_i[p]
 // Every exponent is <= 0 and no quotient of decays is formed. Float32 throughout, FMAs on tiles held in LDS; a chunk's
 // table entry is {request, first row, rows, unused}.
@@ -185,44 +186,78 @@ __global__ void ssm_chunk_states_kernel(float* __restrict__ scratch, const float
   }
 }
 
+// blockIdx = (chunk, group, quarter of i): (C_i . B_j) for the chunk's rows i in the quarter and all j, the same for every
+// head of the group -> pairs [chunks, G, L, L]
+template <typename X>
+__global__ void __launch_bounds__(256)
+ssm_chunk_pairs_kernel(const X* __restrict__ xbc, int64_t ld, float* __restrict__ pairs, const int4* __restrict__ chunks,
+                       int H, int P, int N, int G) {
+  __shared__ float c_s[SSM_L / 4][SSM_PAD];   // [i of the quarter][n of this pass]
+  __shared__ float b_s[SSM_L][SSM_PAD];       // [j][n of this pass]
+  const int chunk = blockIdx.x, group = blockIdx.y, i0 = blockIdx.z * (SSM_L / 4);
+  const int4 entry = chunks[chunk];
+  const int first = entry.y, rows = entry.z;
+  const int64_t b_at = static_cast<int64_t>(H) * P + static_cast<int64_t>(group) * N;
+  const int64_t c_at = b_at + static_cast<int64_t>(G) * N;
+  const int col = threadIdx.x % 64, part = threadIdx.x / 64;      // a thread: j = col, i = i0 + part + 4 r
+  float acc[SSM_L / 16] = {};
+  for (int n0 = 0; n0 < N; n0 += SSM_L) {
+    __syncthreads();
+    for (int i = threadIdx.x; i < SSM_L * SSM_L; i += 256) {
+      const int j = i / SSM_L, n = i % SSM_L;
+      b_s[j][n] = (j < rows && n0 + n < N) ? to_float(xbc[static_cast<int64_t>(first + j) * ld + b_at + n0 + n]) : 0.f;
+    }
+    for (int i = threadIdx.x; i < (SSM_L / 4) * SSM_L; i += 256) {
+      const int r = i / SSM_L, n = i % SSM_L;
+      c_s[r][n] = (i0 + r < rows && n0 + n < N) ? to_float(xbc[static_cast<int64_t>(first + i0 + r) * ld + c_at + n0 + n]) : 0.f;
+    }
+    __syncthreads();
+    for (int n = 0; n < SSM_L; ++n) {
+      const float bv = b_s[col][n];
+#pragma unroll
+      for (int r = 0; r < SSM_L / 16; ++r) acc[r] += c_s[part + 4 * r][n] * bv;
+    }
+  }
+  float* to = pairs + (static_cast<int64_t>(chunk) * G + group) * SSM_L * SSM_L;
+#pragma unroll
+  for (int r = 0; r < SSM_L / 16; ++r) to[(i0 + part + 4 * r) * SSM_L + col] = acc[r];
+}
+
 // blockIdx = (chunk, head, 64 columns p): the chunk's outputs from the state in front of it and its own rows
 template <typename X>
 __global__ void __launch_bounds__(256)
 ssm_chunk_outputs_kernel(const X* __restrict__ xbc, int64_t ld, const X* __restrict__ dt, int64_t ldd,
                          const float* __restrict__ dt_bias, const float* __restrict__ a_log,
-                         const float* __restrict__ skip, const float* __restrict__ scratch, float* __restrict__ out,
-                         const int4* __restrict__ chunks, int H, int P, int N, int G) {
+                         const float* __restrict__ skip, const float* __restrict__ scratch,
+                         const float* __restrict__ pairs, float* __restrict__ out, const int4* __restrict__ chunks, int H,
+                         int P, int N, int G) {
   __shared__ float d_s[SSM_L], l_s[SSM_L];
   __shared__ float a_s[SSM_L][SSM_PAD];     // [i][j]: the pair's weight
-  __shared__ float t_s[SSM_L][SSM_PAD];     // a tile of C [i][n], of B [j][n], of x [j][p] in turn
-  __shared__ float u_s[SSM_L][SSM_PAD];     // a tile of B [j][n], then of the state [n][p]
+  __shared__ float t_s[SSM_L][SSM_PAD];     // a tile of C [i][n], then of x [j][p]
+  __shared__ float u_s[SSM_L][SSM_PAD];     // a tile of the state [n][p]
   const int chunk = blockIdx.x, head = blockIdx.y, p0 = blockIdx.z * 64;
   const int4 entry = chunks[chunk];
   const int first = entry.y, rows = entry.z;
   const int group = head / (H / G);
   chunk_decays(dt, ldd, first, rows, head, dt_bias[head], -expf(a_log[head]), d_s, l_s);
-  const int64_t b_at = static_cast<int64_t>(H) * P + static_cast<int64_t>(group) * N;
-  const int64_t c_at = b_at + static_cast<int64_t>(G) * N;
+  const int64_t c_at = static_cast<int64_t>(H) * P + static_cast<int64_t>(G + group) * N;
   const float* s_in = scratch + (static_cast<int64_t>(chunk) * H + head) * N * P;
   const int col = threadIdx.x % 64, part = threadIdx.x / 64;     // a thread: column col, rows part, part + 4, ...
-  float pair[SSM_L / 4] = {};          // (C_i . B_j) for i = part + 4 r, j = col
+  // the pairs' weights (zero above the diagonal): (C_i . B_j) exp(l_i - l_j) d_j
+  const float* pair = pairs + (static_cast<int64_t>(chunk) * G + group) * SSM_L * SSM_L;
+#pragma unroll
+  for (int r = 0; r < SSM_L / 4; ++r) {
+    const int i = part + 4 * r, j = col;
+    a_s[i][j] = (j <= i && i < rows) ? pair[i * SSM_L + j] * expf(l_s[i] - l_s[j]) * d_s[j] : 0.f;
+  }
   float y[SSM_L / 4] = {};             // outputs for i = part + 4 r, p = col
   for (int n0 = 0; n0 < N; n0 += SSM_L) {
+    // the state's share: sum_n C_i[n] S[n][p] over this pass's n
     __syncthreads();
     for (int i = threadIdx.x; i < SSM_L * SSM_L; i += 256) {
       const int j = i / SSM_L, n = i % SSM_L;
-      const bool in = j < rows && n0 + n < N;
-      t_s[j][n] = in ? to_float(xbc[static_cast<int64_t>(first + j) * ld + c_at + n0 + n]) : 0.f;
-      u_s[j][n] = in ? to_float(xbc[static_cast<int64_t>(first + j) * ld + b_at + n0 + n]) : 0.f;
+      t_s[j][n] = (j < rows && n0 + n < N) ? to_float(xbc[static_cast<int64_t>(first + j) * ld + c_at + n0 + n]) : 0.f;
     }
-    __syncthreads();
-    for (int n = 0; n < SSM_L; ++n) {
-      const float bv = u_s[col][n];
-#pragma unroll
-      for (int r = 0; r < SSM_L / 4; ++r) pair[r] += t_s[part + 4 * r][n] * bv;
-    }
-    // the state's share: sum_n C_i[n] S[n][p] over this pass's n, the state's tile in u_s
-    __syncthreads();
     for (int i = threadIdx.x; i < SSM_L * 64; i += 256) {
       const int n = i / 64, p = i % 64;
       u_s[n][p] = (n0 + n < N && p0 + p < P) ? s_in[static_cast<int64_t>(n0 + n) * P + p0 + p] : 0.f;
@@ -234,13 +269,7 @@ ssm_chunk_outputs_kernel(const X* __restrict__ xbc, int64_t ld, const X* __restr
       for (int r = 0; r < SSM_L / 4; ++r) y[r] += t_s[part + 4 * r][n] * sv;
     }
   }
-  // the pairs' weights (zero above the diagonal), and x into t_s
   __syncthreads();
-#pragma unroll
-  for (int r = 0; r < SSM_L / 4; ++r) {
-    const int i = part + 4 * r, j = col;
-    a_s[i][j] = (j <= i && i < rows) ? pair[r] * expf(l_s[i] - l_s[j]) * d_s[j] : 0.f;
-  }
   for (int i = threadIdx.x; i < SSM_L * 64; i += 256) {
     const int j = i / 64, p = i % 64;
     t_s[j][p] = (j < rows && p0 + p < P) ? to_float(xbc[static_cast<int64_t>(first + j) * ld + head * P + p0 + p]) : 0.f;
@@ -353,14 +382,14 @@ extern "C" int distie_ssm_scan(const void* xbc, int dtype, int64_t ld, const voi
 
 extern "C" int distie_ssm_scan_chunk_rows() { return SSM_L; }
 
-// scratch float32 [chunks, H, N, P], totals float32 [chunks, H]
+// scratch float32 [chunks, H, N, P], totals float32 [chunks, H], pairs float32 [chunks, G, L, L]
 extern "C" int distie_ssm_scan_chunked(const void* xbc, int dtype, int64_t ld, const void* dt, int64_t ldd,
                                        const float* dt_bias, const float* a_log, const float* skip, float* state,
-                                       float* out, float* scratch, float* totals, const void* chunks,
+                                       float* out, float* scratch, float* totals, float* pairs, const void* chunks,
                                        const int32_t* first_chunk, const int32_t* state_slots, int count, int B, int H,
                                        int P, int N, int G, hipStream_t stream) {
   if (B <= 0 || count <= 0) return 0;
-  if (H < 1 || P < 1 || N < 1 || G < 1 || H % G || H > 65535 || ldd < H ||
+  if (H < 1 || P < 1 || N < 1 || G < 1 || H % G || H > 65535 || ldd < H || pairs == nullptr ||
       ld < static_cast<int64_t>(H) * P + 2 * static_cast<int64_t>(G) * N)
     return DISTIE_BAD_ARGUMENT;
   const dim3 grid(count, H, (P + 63) / 64);
@@ -370,9 +399,11 @@ extern "C" int distie_ssm_scan_chunked(const void* xbc, int dtype, int64_t ld, c
     ssm_chunk_sums_kernel<X><<<grid, 256, 0, stream>>>(static_cast<const X*>(xbc), ld, static_cast<const X*>(dt), ldd,
                                                       dt_bias, a_log, scratch, totals, static_cast<const int4*>(chunks),
                                                       H, P, N, G);
+    ssm_chunk_pairs_kernel<X><<<dim3(count, G, 4), 256, 0, stream>>>(static_cast<const X*>(xbc), ld, pairs,
+                                                                    static_cast<const int4*>(chunks), H, P, N, G);
     ssm_chunk_states_kernel<<<dim3(B, H, parts), 256, 0, stream>>>(scratch, totals, state, first_chunk, state_slots, H, size);
     ssm_chunk_outputs_kernel<X><<<grid, 256, 0, stream>>>(static_cast<const X*>(xbc), ld, static_cast<const X*>(dt), ldd,
-                                                         dt_bias, a_log, skip, scratch, out,
+                                                         dt_bias, a_log, skip, scratch, pairs, out,
                                                          static_cast<const int4*>(chunks), H, P, N, G);
   });
   return launch_status();

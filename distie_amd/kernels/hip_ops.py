@@ -333,7 +333,7 @@ class HipOps(Ops):
         o.distie_heads_linear.argtypes = [_P, _I, _I, _P, _I, _P, _I, _I, _I, _I, _I, _P]
         o.distie_head_gate.argtypes = [_P, _I, _I, _I, _P, _I, _L, _P, _I, _I, _I, _P]
         o.distie_ssm_scan.argtypes = [_P, _I, _L, _P, _L, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]
-        o.distie_ssm_scan_chunked.argtypes = [_P, _I, _L, _P, _L, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I,
+        o.distie_ssm_scan_chunked.argtypes = [_P, _I, _L, _P, _L, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I,
                                               _I, _I, _P]
         o.distie_gate_rmsnorm.argtypes = [_P, _P, _I, _F, _P, _I, _L, _P, _I, _I, _I, _I, _I, _P]
         o.distie_glu_mul.argtypes = [_P, _I, _I, _P, _I, _I, _I, _I, _P]
@@ -1660,13 +1660,16 @@ class HipOps(Ops):
         out = torch.empty((T, H * P), dtype=torch.float32, device=self.device)
         if not self.captured and meta.host_cu_q is not None and meta.max_q >= self.SSM_CHUNKED_MIN_ROWS:
             count, packed, scratch = self._scan_chunks(meta, self._ops.distie_ssm_scan_chunk_rows(), H, N, P)
-            key = ("ssm_totals", count, H)
-            totals = meta.scratch.get(key)
-            if totals is None:
-                totals = meta.scratch[key] = torch.empty((count, H), dtype=torch.float32, device=self.device)
+            key = ("ssm_totals", count, H, G)
+            held = meta.scratch.get(key)
+            if held is None:
+                rows = self._ops.distie_ssm_scan_chunk_rows()
+                held = meta.scratch[key] = (torch.empty((count, H), dtype=torch.float32, device=self.device),
+                                            torch.empty((count, G, rows, rows), dtype=torch.float32, device=self.device))
+            totals, pairs = held
             _check(self._ops.distie_ssm_scan_chunked(
                 x_ptr, _code(xbc), ld, d_ptr, ldd, dt_bias.data_ptr(), a_log.data_ptr(), skip.data_ptr(),
-                state.data_ptr(), out.data_ptr(), scratch.data_ptr(), totals.data_ptr(), packed.data_ptr(),
+                state.data_ptr(), out.data_ptr(), scratch.data_ptr(), totals.data_ptr(), pairs.data_ptr(), packed.data_ptr(),
                 packed.data_ptr() + 16 * count, meta.state_slots.data_ptr(), count, meta.num_requests, H, P, N, G,
                 self._stream()), "ssm_scan_chunked")
             _mark_written(state)
