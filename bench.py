@@ -279,21 +279,21 @@ def sekazen_config(size):
 
 
 def dufelix_config(size):
-    """Groups of four layers: two of latent attention (a latent of 192 and a rotated key part of 64 for all heads,
-    queries through a latent of three eighths of the width, a sink for each head), a state-space layer (heads of 64
-    channels on twice the width, a state of 128 rows, four taps) and one of grouped-query attention with half of every
-    head turned and a gate for each head; norms on both sides of every sub-layer, gelu-gated dense feed-forwards."""
+    """Groups of four layers: latent attention (a latent of 192 and a rotated key part of 64 for all heads, queries
+    through a latent of three eighths of the width, a sink for each head), a state-space layer (heads of 64 channels on
+    twice the width, a state of 128 rows, four taps), latent attention again, and grouped-query attention with half of
+    every head turned and a gate for each head; norms on both sides of every sub-layer, gelu-gated dense feed-forwards."""
     z = DESIGN_SIZES[size]
     stretch = {"factor": 8.0, "original": 1024, "fast": 32.0, "slow": 1.0}
     layers = []
     for i in range(z["layers"]):
         mlp = {"kind": "dense", "ff": z["ff"]}
-        if i % 4 < 2:
+        if i % 4 in (0, 2):
             mixer = {"heads": z["heads"], "dim": z["dim"], "rot_dim": 64, "vdim": z["dim"], "kv_rank": 192,
                      "q_rank": 3 * z["width"] // 8, "scale": (z["dim"] + 64) ** -0.5,
                      "rot": {"base": 10000.0, "dims": 64, "scaling": stretch}}
             layers.append({"type": "latent_attention", "mixer": mixer, "mlp": mlp})
-        elif i % 4 == 2:
+        elif i % 4 == 1:
             mixer = {"heads": 2 * z["width"] // 64, "vdim": 64, "state": 128, "groups": 1, "conv": 4, "norm_groups": 1}
             layers.append({"type": "mamba2", "mixer": mixer, "mlp": mlp})
         else:

@@ -290,10 +290,12 @@ ssm_chunk_outputs_kernel(const X* __restrict__ xbc, int64_t ld, const X* __restr
 // out = (x * gate) / sqrt(mean((x * gate)^2) + eps) * weight, the mean over each run of N columns of a row by itself
 // (`groups` runs side by side in a row of x, of the gates and of out); gate = g * sigmoid(g) (`silu`) or sigmoid(g);
 // the weight is each column's own, [groups * N]. The gate stands in front of the norm. One block a (row, run).
-template <typename W, typename G, typename O>
+// STAGED: the gated values of the run wait in LDS between the two walks, so x and the gates are read once.
+template <bool STAGED, typename W, typename G, typename O>
 __global__ void gate_rmsnorm_kernel(const float* __restrict__ x, const W* __restrict__ weight, float eps,
                                     const G* __restrict__ gates, int64_t ldg, O* __restrict__ out, int N, int groups,
                                     int silu) {
+  extern __shared__ float held[];
   __shared__ float scratch[16];
   const int64_t t = blockIdx.x;
   const int64_t at = static_cast<int64_t>(blockIdx.y) * N;
@@ -303,13 +305,19 @@ __global__ void gate_rmsnorm_kernel(const float* __restrict__ x, const W* __rest
   for (int c = threadIdx.x; c < N; c += blockDim.x) {
     const float z = to_float(g[c]);
     const float v = row[c] * (silu ? z * sigmoidf(z) : sigmoidf(z));
+    if constexpr (STAGED) held[c] = v;
     sq += v * v;
   }
   sq = block_sum(sq, scratch);
   const float scale = 1.f / sqrtf(sq / N + eps);
   for (int c = threadIdx.x; c < N; c += blockDim.x) {
-    const float z = to_float(g[c]);
-    const float v = row[c] * (silu ? z * sigmoidf(z) : sigmoidf(z));
+    float v;
+    if constexpr (STAGED) {
+      v = held[c];                       // (written by this same thread)
+    } else {
+      const float z = to_float(g[c]);
+      v = row[c] * (silu ? z * sigmoidf(z) : sigmoidf(z));
+    }
     out[t * N * groups + at + c] = from_float<O>(v * scale * to_float(weight[at + c]));
   }
 }
@@ -416,9 +424,15 @@ extern "C" int distie_gate_rmsnorm(const float* x, const void* weight, int w_dty
   if (N < 1 || groups < 1 || groups > 65535 || gates == nullptr || ldg < static_cast<int64_t>(N) * groups)
     return DISTIE_BAD_ARGUMENT;
   const int threads = N >= 1024 ? 1024 : (N >= 512 ? 512 : (N >= 256 ? 256 : (N >= 128 ? 128 : 64)));
-  DISTIE_DISPATCH(w_dtype, W, DISTIE_DISPATCH(g_dtype, G, DISTIE_DISPATCH(out_dtype, O,
-      gate_rmsnorm_kernel<W, G, O><<<dim3(T, groups), threads, 0, stream>>>(
-          x, static_cast<const W*>(weight), eps, static_cast<const G*>(gates), ldg, static_cast<O*>(out), N, groups, silu))));
+  if (N <= 12288) {
+    DISTIE_DISPATCH(w_dtype, W, DISTIE_DISPATCH(g_dtype, G, DISTIE_DISPATCH(out_dtype, O,
+        gate_rmsnorm_kernel<true, W, G, O><<<dim3(T, groups), threads, sizeof(float) * N, stream>>>(
+            x, static_cast<const W*>(weight), eps, static_cast<const G*>(gates), ldg, static_cast<O*>(out), N, groups, silu))));
+  } else {
+    DISTIE_DISPATCH(w_dtype, W, DISTIE_DISPATCH(g_dtype, G, DISTIE_DISPATCH(out_dtype, O,
+        gate_rmsnorm_kernel<false, W, G, O><<<dim3(T, groups), threads, 0, stream>>>(
+            x, static_cast<const W*>(weight), eps, static_cast<const G*>(gates), ldg, static_cast<O*>(out), N, groups, silu))));
+  }
   return launch_status();
 }
 

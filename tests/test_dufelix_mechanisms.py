@@ -109,7 +109,7 @@ def dufelix_mixer(cfg):
 @pytest.mark.parametrize("sizes", [dict(heads=3, dim=12, rot_dim=8, vdim=20, kv_rank=24, q_rank=28),
                                    dict(heads=1, dim=16, rot_dim=16, vdim=16, kv_rank=16, q_rank=16, scaled=False),
                                    dict(heads=5, dim=10, rot_dim=6, vdim=14, kv_rank=18, q_rank=22),
-                                   dict(heads=4, dim=32, rot_dim=32, vdim=32, kv_rank=96, q_rank=64),
+                                   dict(heads=4, dim=32, rot_dim=32, vdim=32, kv_rank=88, q_rank=64),
                                    dict(heads=2, dim=24, rot_dim=16, vdim=40, kv_rank=176, q_rank=48)])
 def test_latent_attention_alone(ops, sizes):
     """Latent attention as a part over batches in steps: the cached latent and rotated key part serve every head, the
@@ -159,7 +159,7 @@ def test_latent_cache_holds_the_latent_and_one_turned_part(ops):
 @pytest.mark.parametrize("sizes", [dict(heads=4, kv_heads=2, dim=16, vdim=24, dims=8),
                                    dict(heads=2, kv_heads=2, dim=32, vdim=32, dims=0),
                                    dict(heads=5, kv_heads=1, dim=20, vdim=12, dims=6),
-                                   dict(heads=4, kv_heads=2, dim=96, vdim=48, dims=48),
+                                   dict(heads=6, kv_heads=3, dim=80, vdim=40, dims=32),
                                    dict(heads=1, kv_heads=1, dim=64, vdim=64, dims=64, scaled=False)])
 def test_attention_with_a_gate_for_each_head(ops, sizes):
     layer = du.attention(scale=0.3, base=200.0, **sizes)
@@ -241,7 +241,7 @@ def build_state(H, N, P):
 
 
 def test_gate_in_front_of_the_grouped_norm(ops):
-    for N, groups in ((24, 1), (60, 3), (288, 2), (2048, 8)):
+    for N, groups in ((24, 1), (60, 3), (272, 2), (2048, 8)):
         for dtype in act_types(ops):
             x, z = rnd(9, N, seed=1, scale=3.0), rnd(9, N + 8, seed=2).to(dtype)
             weight = (1 + rnd(N, seed=3, scale=0.3)).to(dtype)
@@ -280,7 +280,7 @@ def test_products_by_head(ops):
     """Every head's own product, for few rows and for many, with inputs and results that lie apart in wider rows."""
     dev = lambda t: t.to(ops.device)
     for T in (1, 5, 16, 17, 150):
-        for H, N, K, lx, lo in ((3, 24, 12, 20, 32), (1, 16, 16, 16, 16), (5, 18, 10, 16, 24), (4, 80, 96, 128, 80)):
+        for H, N, K, lx, lo in ((3, 24, 12, 20, 32), (1, 16, 16, 16, 16), (5, 18, 10, 16, 24), (4, 72, 104, 128, 72)):
             for dtype in act_types(ops):
                 x, w = rnd(T, H * lx, seed=1).to(dtype), rnd(H, N, K, seed=2, scale=0.3).to(dtype)
                 got = ops.heads_linear(dev(x), dev(w), lx, lo).float().cpu().view(T, H, lo)
@@ -293,7 +293,7 @@ def test_convolution_with_bias_and_activation(ops):
     """The short convolution over column views with a bias and silu behind it, its state carried over steps of one
     row and of more rows than it has taps, and of fewer."""
     lengths, cuts = (11, 4, 7), ((2, 1, 7), (1, 1, 0), (5, 2, 0), (3, 0, 0))
-    for taps, N in ((1, 24), (3, 40), (4, 56), (4, 416)):
+    for taps, N in ((1, 24), (3, 40), (4, 56), (4, 424)):
         for dtype in act_types(ops):
             from distie_amd.parts import FixedState, TensorDecl
 
