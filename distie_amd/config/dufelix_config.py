@@ -4,8 +4,8 @@ config.json names everything that can differ between models of the design:
 
     architecture "Dufelix", vocab, width, norm.eps, embedding.scale, and `layers`, one entry a layer: `type`
     ("attention" | "latent_attention" | "mamba2"), `mixer` (its sizes), `mlp` ({"kind": "dense", "ff": n} or null) and,
-    optionally, `weights_of`: an earlier layer whose tensors (mixer, feed-forward, norms) this layer uses, with a cache
-    or state of its own.
+    optionally, `weights_of`: another layer whose tensors (mixer, feed-forward, norms) this layer uses, with a cache
+    or state of its own (its type and sizes are that layer's; an entry may repeat them).
 
     attention mixer: heads, kv_heads, dim, vdim, rot {base, dims, scaling {factor, original, fast, slow}}, scale.
     latent_attention mixer: heads, dim, rot_dim, vdim, kv_rank, q_rank, rot (as above, dims = rot_dim), scale.
@@ -81,12 +81,14 @@ class DufelixConfig:
                 raise ConfigError(f"{where}: unknown layer type {kind!r}")
             source = layer.get("weights_of")
             if source is not None:
-                source = int(source)
-                if not 0 <= source < i or layers[source].get("weights_of") is not None:
-                    raise ConfigError(f"{where}: weights_of must name an earlier layer with tensors of its own")
-                theirs = layers[source]
-                if theirs.get("type") != kind or theirs.get("mixer") != layer.get("mixer") or theirs.get("mlp") != layer.get("mlp"):
-                    raise ConfigError(f"{where}: a layer that uses layer {source}'s tensors has its type and sizes")
+                owner = cls._owner(layers, i)
+                theirs = layers[owner]
+                if theirs.get("type") != kind:
+                    raise ConfigError(f"{where}: a layer that uses layer {owner}'s tensors has its type")
+                for key in ("mixer", "mlp"):
+                    if key in layer and cls._sizes(layer[key]) != cls._sizes(theirs.get(key)):
+                        raise ConfigError(f"{where}: a layer that uses layer {owner}'s tensors has its sizes")
+                continue                                         # (its sizes are the owner's, checked there)
             m = layer.get("mixer")
             if kind == "attention":
                 heads, kv_heads = _need(m, "heads", int, where), _need(m, "kv_heads", int, where)
@@ -127,6 +129,27 @@ class DufelixConfig:
                     raise ConfigError(f"{where}: mlp.ff must be >= 1")
         return cls(data=dict(data), max_positions=int(data.get("max_positions") or DEFAULT_MAX_POSITIONS))
 
+    @staticmethod
+    def _owner(layers, i: int) -> int:
+        """The layer whose tensors layer i uses: itself, or where its chain of `weights_of` ends."""
+        seen = {i}
+        while layers[i].get("weights_of") is not None:
+            j = layers[i]["weights_of"]
+            if isinstance(j, bool) or not isinstance(j, int) or not 0 <= j < len(layers) or j in seen:
+                raise ConfigError(f"layer {i}: weights_of must name another layer of the model")
+            seen.add(j)
+            i = j
+        return i
+
+    @staticmethod
+    def _sizes(value):
+        """A mixer's or feed-forward's entry as numbers compare, whatever way a file wrote them (1 and 1.0 are one size)."""
+        if isinstance(value, Mapping):
+            return {k: DufelixConfig._sizes(v) for k, v in value.items()}
+        if isinstance(value, (int, float)) and not isinstance(value, bool):
+            return float(value)
+        return value
+
     def to_dict(self) -> dict:
         return dict(self.data)
 
@@ -135,9 +158,9 @@ class DufelixConfig:
         data = dict(self.data)
         layers = []
         for i, layer in enumerate(data["layers"]):
-            name = f"l{int(layer['weights_of']) if layer.get('weights_of') is not None else i}.mix.dq"
-            if layer.get("type") == "latent_attention" and layer["mixer"].get("q_rank") is None and \
-                    name in shapes and len(shapes[name]) == 2:
+            name = f"l{self._owner(data['layers'], i)}.mix.dq"
+            if layer.get("type") == "latent_attention" and isinstance(layer.get("mixer"), Mapping) and \
+                    layer["mixer"].get("q_rank") is None and name in shapes and len(shapes[name]) == 2:
                 layer = dict(layer, mixer=dict(layer["mixer"], q_rank=int(shapes[name][0])))
             layers.append(layer)
         data["layers"] = layers
@@ -172,9 +195,11 @@ class DufelixConfig:
         width, eps = self.hidden_size, float(data["norm"]["eps"])
         norm = lambda base, name: PartSpec("rmsnorm", base, {"size": width, "eps": eps, "weight_name": name})
         layers = []
-        for i, layer in enumerate(data["layers"]):
-            source = layer.get("weights_of")
-            base = f"l{i if source is None else int(source)}."
+        for i, entry in enumerate(data["layers"]):
+            owner = self._owner(data["layers"], i)
+            source = None if owner == i else owner
+            layer = data["layers"][owner]                    # a layer that uses another's tensors is described by it
+            base = f"l{owner}."
             parts = {"mixer": self._mixer(layer["type"], layer["mixer"], base + "mix.", i),
                      "mixer_norm": norm(base, "norm1"), "mixer_post_norm": norm(base, "norm1b")}
             mlp = layer.get("mlp")

@@ -26,18 +26,20 @@ class Model:
         self.embed = build_part("embedding", spec.embedding)
         # a layer that uses an earlier layer's tensors is that layer's block once more: one set of parts and weights,
         # and (the cache being declared and addressed by layer) pages and state of its own
-        self.blocks = []
+        self.blocks = [None] * len(spec.layers)
         for index, layer in enumerate(spec.layers):
             if layer.weights_of is None:
-                self.blocks.append(build_part("block", layer.block, layer.parts))
+                self.blocks[index] = build_part("block", layer.block, layer.parts)
+        for index, layer in enumerate(spec.layers):
+            if layer.weights_of is None:
                 continue
             source = int(layer.weights_of)
-            if not 0 <= source < index or spec.layers[source].weights_of is not None:
-                raise ValueError(f"layer {index} uses the tensors of layer {source}, which must be an earlier layer with "
-                                 f"tensors of its own")
+            if not 0 <= source < len(spec.layers) or spec.layers[source].weights_of is not None:
+                raise ValueError(f"layer {index} uses the tensors of layer {source}, which must be a layer with tensors "
+                                 f"of its own")
             if (layer.block, dict(layer.parts)) != (spec.layers[source].block, dict(spec.layers[source].parts)):
                 raise ValueError(f"layer {index} uses the tensors of layer {source} and must be described like it")
-            self.blocks.append(self.blocks[source])
+            self.blocks[index] = self.blocks[source]
         self.final_norm = build_part("norm", spec.final_norm)
         self.position = build_part("position", spec.position) if spec.position is not None else None
         self.lm_head = build_part("head", spec.head)

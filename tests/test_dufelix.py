@@ -135,13 +135,22 @@ def test_configuration_and_tensors():
     assert {n: tuple(s.shape) for n, s in Model.declare(config.model_spec()).items()} == du.tensor_shapes(MIXED)
     with pytest.raises(ConfigError):
         config_from_dict(bare).model_spec()
+    # a layer may name a layer that itself names another (the tensors are the last one's), or a later layer, and may
+    # leave out the sizes that it has from there
+    chain = {**MIXED, "layers": [du.mamba(), du.mamba(weights_of=0), {"type": "mamba2", "weights_of": 1},
+                                 {"type": "attention", "weights_of": 4}, du.attention()]}
+    spec = config_from_dict(chain).model_spec()
+    assert [layer.weights_of for layer in spec.layers] == [None, 0, 0, 4, None]
+    model = Model(spec)
+    assert model.blocks[2] is model.blocks[0] and model.blocks[3] is model.blocks[4]
+    assert {n for n in Model.declare(spec)} == set(du.tensor_shapes({**MIXED, "layers": [du.mamba(), du.mamba(weights_of=0),
+                                                                    du.mamba(weights_of=0), du.attention(weights_of=4), du.attention()]}))
     for broken in ({**MIXED, "layers": [du.attention(heads=3, kv_heads=2)]},
                    {**MIXED, "layers": [du.attention(dims=18, dim=16)]},
                    {**MIXED, "layers": [du.latent(rot_dim=7)]},
                    {**MIXED, "layers": [du.mamba(heads=4, groups=3)]},
                    {**MIXED, "layers": [du.mamba(heads=3, vdim=5, groups=1, norm_groups=2)]},
                    {**MIXED, "layers": [du.mamba(), du.mamba(weights_of=1)]},
-                   {**MIXED, "layers": [du.mamba(), du.mamba(weights_of=0), du.mamba(weights_of=1)]},
                    {**MIXED, "layers": [du.mamba(), du.mamba(weights_of=0, state=16)]},
                    {**MIXED, "layers": [du.mamba(), du.latent(weights_of=0)]},
                    {**MIXED, "layers": [du.mamba(mlp={"kind": "moe", "ff": 8})]},
