@@ -1,4 +1,4 @@
-// Attention over the paged cache for one head size (compile with -DDISTIE_HEAD_DIM=<even size up to 256>; the
+// Attention over the paged cache for one head size (compile with -DDISTIE_HEAD_DIM=<even size up to 1024>; the
 // matrix-core kernels exist for multiples of 16 only, the wave-per-token kernel for every even size).
 //
 // out[t, h] = softmax_j(q[t, h] . k[j, h / G] * scale) v[j, h / G] over the keys j that token t may see:
@@ -19,10 +19,11 @@
 #ifndef DISTIE_HEAD_DIM
 #error "compile with -DDISTIE_HEAD_DIM=<head size>"
 #endif
-#if DISTIE_HEAD_DIM % 2 != 0 || DISTIE_HEAD_DIM < 2 || DISTIE_HEAD_DIM > 256
-#error "head size must be even and at most 256"
+#if DISTIE_HEAD_DIM % 2 != 0 || DISTIE_HEAD_DIM < 2 || DISTIE_HEAD_DIM > 1024
+#error "head size must be even and at most 1024"
 #endif
-#define DISTIE_MATRIX_CORE_ATTENTION (DISTIE_HEAD_DIM % 16 == 0)
+// (beyond 256 the matrix-core kernels' tiles no longer fit their registers and LDS: the wave-per-token kernel serves)
+#define DISTIE_MATRIX_CORE_ATTENTION (DISTIE_HEAD_DIM % 16 == 0 && DISTIE_HEAD_DIM <= 256)
 
 constexpr int D = DISTIE_HEAD_DIM;
 constexpr int DIMS_PER_LANE = (D + DISTIE_WAVE - 1) / DISTIE_WAVE;

@@ -6,7 +6,7 @@ Four kinds of shared library, all built from the sources beside this file:
 * `ops`   - the HIP kernels that do not depend on the head size (hipcc, gfx950);
 * `library` - the calls of the vendor's matrix-product library for large products (hipcc, linked with hipBLASLt);
 * `attn_d<D>` - the attention kernels for head size D (hipcc, `-DDISTIE_HEAD_DIM=D`; the matrix-core
-  kernels for multiples of 16, the wave-per-token kernel for every even size).
+  kernels for multiples of 16 up to 256, the wave-per-token kernel for every even size up to 1024).
 
 A library's file name carries a hash of its sources and flags, so a stale build is never
 loaded. Libraries live in `distie_amd/_lib/` (in-tree); if that folder cannot be written,
@@ -74,8 +74,8 @@ def _spec(name: str):
         return list(LIBRARY_SOURCES), _hipcc(), list(HIP_FLAGS)
     if name.startswith("attn_d"):
         dim = int(name[len("attn_d"):])
-        if dim < 2 or dim > 256 or dim % 2:
-            raise BuildError(f"attention kernels are built for even head sizes up to 256, not {dim}")
+        if dim < 2 or dim > 1024 or dim % 2:
+            raise BuildError(f"attention kernels are built for even head sizes up to 1024, not {dim}")
         return list(ATTN_SOURCES), _hipcc(), list(HIP_FLAGS) + [f"-DDISTIE_HEAD_DIM={dim}"]
     raise BuildError(f"no native library named {name}")
 
@@ -195,7 +195,7 @@ def ensure(name: str) -> Path:
     return build(name, force=False)
 
 
-DEFAULT_HEAD_DIMS = (16, 32, 40, 48, 64, 80, 96, 112, 128, 192, 256)
+DEFAULT_HEAD_DIMS = (16, 32, 40, 48, 64, 80, 96, 112, 128, 192, 256, 288)
 
 
 def build_all(head_dims=DEFAULT_HEAD_DIMS, force: bool = True) -> List[Path]:

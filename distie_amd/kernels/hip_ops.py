@@ -221,6 +221,10 @@ class HipOps(Ops):
     # length are cut as before). Everywhere else it is level or behind (32 requests: 30 -> 33 us).
     DECODE_SHARED_BELOW = 0.8
     DECODE_MAX_RUNS = 256
+    # the matrix-core attention kernels take heads up to 256; wider ones (a latent that all heads share) run on the
+    # wave-per-token kernel, in either precision
+    LARGEST_MATRIX_CORE_HEAD = 256
+    LARGEST_HEAD = 1024
 
     def __init__(self, device="cuda:0", packed_weights=True) -> None:
         """`packed_weights` (True, False, or the roles that get one, as the parts name them in
@@ -365,8 +369,8 @@ class HipOps(Ops):
     def attention_library(self, head_dim: int) -> ctypes.CDLL:
         lib = self._attn.get(head_dim)
         if lib is None:
-            if head_dim % 2 or not 2 <= head_dim <= 256:
-                raise KernelError(f"attention kernels take even head sizes up to 256, not {head_dim}")
+            if head_dim % 2 or not 2 <= head_dim <= self.LARGEST_HEAD:
+                raise KernelError(f"attention kernels take even head sizes up to {self.LARGEST_HEAD}, not {head_dim}")
             lib = ctypes.CDLL(str(build.ensure(f"attn_d{head_dim}")))
             lib.distie_attention_generic.argtypes = [_P, _I, _L, _P, _P, _I, _P, _P, _P, _I, _P, _P,
                                                      _I, _I, _I, _I, _F, _I, _P, _F, _P, _P]
@@ -945,7 +949,7 @@ class HipOps(Ops):
                     raise KernelError(f"paged_attention: {name} must be float32 [num_heads]")
         sinks_ptr = sinks.data_ptr() if sinks is not None else None
         bf16 = qkv.dtype == torch.bfloat16 and k_cache.dtype == torch.bfloat16
-        if plain and bf16 and meta.block_size % 16 == 0 and head_dim % 16 == 0:
+        if plain and bf16 and meta.block_size % 16 == 0 and head_dim % 16 == 0 and head_dim <= self.LARGEST_MATRIX_CORE_HEAD:
             # how the step is launched, and its buffers for partial results, are the same for every layer
             # with these sizes: worked out once per step (the layers run one after the other, so they can
             # share the buffers)

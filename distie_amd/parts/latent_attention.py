@@ -18,7 +18,8 @@ Only c and the rotated r are kept, and attention runs on them directly: q_h . (W
 the query of head h taken to the latent's space every head reads the same cached vector (c, rot(r)) as its key and c as
 its value, which is attention with one key/value head of size kv_rank + rot_dim, and W_uv,h is applied to the weighted
 sum of the c's afterwards. The kernels are the ones every attention layer uses (one key/value head, H query heads on
-it); their head size is kv_rank + rot_dim rounded up to what they take, so that sum is bounded by their largest head.
+it); their head size is kv_rank + rot_dim rounded up to what they take, so that sum is bounded by their largest head
+(beyond the matrix-core kernels' 256 the wave-per-token kernel serves, slowly).
 The two down-projections are one matrix product (their weights are stacked at load), both norms, the rotation of r and
 the cache write one kernel.
 """
@@ -35,7 +36,7 @@ from .attention import PagedKV, context_classes
 from .base import Mixer, ParamSpec, build_part, register_part
 from .conv_attention import padded_head_dim
 
-LARGEST_HEAD = 256          # what the attention kernels take
+LARGEST_HEAD = 1024         # what the attention kernels take (the matrix-core ones up to 256, the wave-per-token one beyond)
 
 
 class LatentAttention(Mixer):

@@ -110,11 +110,12 @@ def dufelix_mixer(cfg):
                                    dict(heads=1, dim=16, rot_dim=16, vdim=16, kv_rank=16, q_rank=16, scaled=False),
                                    dict(heads=5, dim=10, rot_dim=6, vdim=14, kv_rank=18, q_rank=22),
                                    dict(heads=4, dim=32, rot_dim=32, vdim=32, kv_rank=88, q_rank=64),
-                                   dict(heads=2, dim=24, rot_dim=16, vdim=40, kv_rank=176, q_rank=48)])
+                                   dict(heads=2, dim=24, rot_dim=16, vdim=40, kv_rank=176, q_rank=48),
+                                   dict(heads=3, dim=16, rot_dim=8, vdim=24, kv_rank=280, q_rank=40)])
 def test_latent_attention_alone(ops, sizes):
     """Latent attention as a part over batches in steps: the cached latent and rotated key part serve every head, the
-    sink joins the denominator, neighbouring dimensions are turned. Sizes that fit no tile, all equal, and a latent
-    wider than the kernels' most common head."""
+    sink joins the denominator, neighbouring dimensions are turned. Sizes that fit no tile, all equal, a latent
+    wider than the kernels' most common head, and one beyond the matrix-core kernels' largest."""
     layer = du.latent(scale=0.3, base=200.0, **sizes)
     mixer_case(ops, layer, dufelix_mixer, lambda h, w, p, m, pos, eps: plain.latent_attention(h, w, p, m, pos, eps),
                LENGTHS, CUTS, slack=2.0)
