@@ -101,6 +101,12 @@ ssm_scan_kernel(const X* __restrict__ xbc, int64_t ld, const X* __restrict__ dt,
 constexpr int SSM_L = 64;
 constexpr int SSM_PAD = SSM_L + 1;
 
+// The products of the chunks' tiles run on v_mfma_f32_32x32x2_f32 (float32 operands, products and sums): a lane gives
+// A[row = lane % 32][k = lane / 32] and B[k = lane / 32][column = lane % 32], both read from LDS tiles whose rows are an
+// odd number of words apart, and holds, in register v, the sum for row tile_row(v, lane) and column lane % 32.
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float ssm_floatx16;
+__device__ __forceinline__ int tile_row(int v, int lane) { return 8 * (v / 4) + 4 * (lane / 32) + v % 4; }
+
 // d_j and l_j of a chunk's rows for one head, into LDS (thread 0 adds the logarithms in order)
 template <typename X>
 __device__ __forceinline__ void chunk_decays(const X* __restrict__ dt, int64_t ldd, int first, int rows, int head,
@@ -125,7 +131,7 @@ ssm_chunk_sums_kernel(const X* __restrict__ xbc, int64_t ld, const X* __restrict
                       const float* __restrict__ dt_bias, const float* __restrict__ a_log, float* __restrict__ scratch,
                       float* __restrict__ totals, const int4* __restrict__ chunks, int H, int P, int N, int G) {
   __shared__ float d_s[SSM_L], l_s[SSM_L];
-  __shared__ float x_s[SSM_L][64];          // [row][p], times the row's factor
+  __shared__ float x_s[SSM_L][SSM_PAD];     // [row][p], times the row's factor
   __shared__ float b_s[SSM_L][SSM_PAD];     // [row][n of this pass]
   const int chunk = blockIdx.x, head = blockIdx.y, p0 = blockIdx.z * 64;
   const int4 entry = chunks[chunk];
@@ -142,7 +148,9 @@ ssm_chunk_sums_kernel(const X* __restrict__ xbc, int64_t ld, const X* __restrict
   }
   const int64_t b_at = static_cast<int64_t>(H) * P + static_cast<int64_t>(group) * N;
   float* u = scratch + (static_cast<int64_t>(chunk) * H + head) * N * P;
-  const int p = threadIdx.x % 64, part = threadIdx.x / 64;       // a thread: column p, rows n = part, part + 4, ...
+  // a wave: 32 rows n by 32 columns p of the pass's 64 x 64, on float32 matrix products over the rows j
+  const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+  const int nb = 32 * (wave / 2), pb = 32 * (wave % 2);
   for (int n0 = 0; n0 < N; n0 += SSM_L) {
     __syncthreads();
     for (int i = threadIdx.x; i < SSM_L * SSM_L; i += 256) {
@@ -150,16 +158,14 @@ ssm_chunk_sums_kernel(const X* __restrict__ xbc, int64_t ld, const X* __restrict
       b_s[j][n] = (j < rows && n0 + n < N) ? to_float(xbc[static_cast<int64_t>(first + j) * ld + b_at + n0 + n]) : 0.f;
     }
     __syncthreads();
-    float acc[SSM_L / 4] = {};
-    for (int j = 0; j < rows; ++j) {
-      const float xv = x_s[j][p];
+    ssm_floatx16 acc = {};
+    for (int j = 0; j < SSM_L; j += 2)
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(b_s[j + lane / 32][nb + lane % 32], x_s[j + lane / 32][pb + lane % 32],
+                                                 acc, 0, 0, 0);
 #pragma unroll
-      for (int r = 0; r < SSM_L / 4; ++r) acc[r] += b_s[j][part + 4 * r] * xv;
-    }
-#pragma unroll
-    for (int r = 0; r < SSM_L / 4; ++r) {
-      const int n = n0 + part + 4 * r;
-      if (n < N && p0 + p < P) u[static_cast<int64_t>(n) * P + p0 + p] = acc[r];
+    for (int v = 0; v < 16; ++v) {
+      const int n = n0 + nb + tile_row(v, lane), pc = p0 + pb + lane % 32;
+      if (n < N && pc < P) u[static_cast<int64_t>(n) * P + pc] = acc[v];
     }
   }
 }
@@ -186,41 +192,38 @@ __global__ void ssm_chunk_states_kernel(float* __restrict__ scratch, const float
   }
 }
 
-// blockIdx = (chunk, group, quarter of i): (C_i . B_j) for the chunk's rows i in the quarter and all j, the same for every
-// head of the group -> pairs [chunks, G, L, L]
+// blockIdx = (chunk, group): (C_i . B_j) for the chunk's rows i and j, the same for every head of the group
+// -> pairs [chunks, G, L, L]. A wave: 32 rows i by 32 columns j.
 template <typename X>
 __global__ void __launch_bounds__(256)
 ssm_chunk_pairs_kernel(const X* __restrict__ xbc, int64_t ld, float* __restrict__ pairs, const int4* __restrict__ chunks,
                        int H, int P, int N, int G) {
-  __shared__ float c_s[SSM_L / 4][SSM_PAD];   // [i of the quarter][n of this pass]
+  __shared__ float c_s[SSM_L][SSM_PAD];       // [i][n of this pass]
   __shared__ float b_s[SSM_L][SSM_PAD];       // [j][n of this pass]
-  const int chunk = blockIdx.x, group = blockIdx.y, i0 = blockIdx.z * (SSM_L / 4);
+  const int chunk = blockIdx.x, group = blockIdx.y;
   const int4 entry = chunks[chunk];
   const int first = entry.y, rows = entry.z;
   const int64_t b_at = static_cast<int64_t>(H) * P + static_cast<int64_t>(group) * N;
   const int64_t c_at = b_at + static_cast<int64_t>(G) * N;
-  const int col = threadIdx.x % 64, part = threadIdx.x / 64;      // a thread: j = col, i = i0 + part + 4 r
-  float acc[SSM_L / 16] = {};
+  const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+  const int ib = 32 * (wave / 2), jb = 32 * (wave % 2);
+  ssm_floatx16 acc = {};
   for (int n0 = 0; n0 < N; n0 += SSM_L) {
     __syncthreads();
     for (int i = threadIdx.x; i < SSM_L * SSM_L; i += 256) {
       const int j = i / SSM_L, n = i % SSM_L;
-      b_s[j][n] = (j < rows && n0 + n < N) ? to_float(xbc[static_cast<int64_t>(first + j) * ld + b_at + n0 + n]) : 0.f;
-    }
-    for (int i = threadIdx.x; i < (SSM_L / 4) * SSM_L; i += 256) {
-      const int r = i / SSM_L, n = i % SSM_L;
-      c_s[r][n] = (i0 + r < rows && n0 + n < N) ? to_float(xbc[static_cast<int64_t>(first + i0 + r) * ld + c_at + n0 + n]) : 0.f;
+      const bool in = j < rows && n0 + n < N;
+      b_s[j][n] = in ? to_float(xbc[static_cast<int64_t>(first + j) * ld + b_at + n0 + n]) : 0.f;
+      c_s[j][n] = in ? to_float(xbc[static_cast<int64_t>(first + j) * ld + c_at + n0 + n]) : 0.f;
     }
     __syncthreads();
-    for (int n = 0; n < SSM_L; ++n) {
-      const float bv = b_s[col][n];
-#pragma unroll
-      for (int r = 0; r < SSM_L / 16; ++r) acc[r] += c_s[part + 4 * r][n] * bv;
-    }
+    for (int n = 0; n < SSM_L; n += 2)
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(c_s[ib + lane % 32][n + lane / 32], b_s[jb + lane % 32][n + lane / 32],
+                                                 acc, 0, 0, 0);
   }
   float* to = pairs + (static_cast<int64_t>(chunk) * G + group) * SSM_L * SSM_L;
 #pragma unroll
-  for (int r = 0; r < SSM_L / 16; ++r) to[(i0 + part + 4 * r) * SSM_L + col] = acc[r];
+  for (int v = 0; v < 16; ++v) to[(ib + tile_row(v, lane)) * SSM_L + jb + lane % 32] = acc[v];
 }
 
 // blockIdx = (chunk, head, 64 columns p): the chunk's outputs from the state in front of it and its own rows
@@ -250,9 +253,11 @@ ssm_chunk_outputs_kernel(const X* __restrict__ xbc, int64_t ld, const X* __restr
     const int i = part + 4 * r, j = col;
     a_s[i][j] = (j <= i && i < rows) ? pair[i * SSM_L + j] * expf(l_s[i] - l_s[j]) * d_s[j] : 0.f;
   }
-  float y[SSM_L / 4] = {};             // outputs for i = part + 4 r, p = col
+  // a wave: 32 rows i by 32 columns p of the outputs
+  const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+  const int ib = 32 * (wave / 2), pb = 32 * (wave % 2);
+  ssm_floatx16 y = {};                 // the state's share: sum_n C_i[n] S[n][p]
   for (int n0 = 0; n0 < N; n0 += SSM_L) {
-    // the state's share: sum_n C_i[n] S[n][p] over this pass's n
     __syncthreads();
     for (int i = threadIdx.x; i < SSM_L * SSM_L; i += 256) {
       const int j = i / SSM_L, n = i % SSM_L;
@@ -263,11 +268,9 @@ ssm_chunk_outputs_kernel(const X* __restrict__ xbc, int64_t ld, const X* __restr
       u_s[n][p] = (n0 + n < N && p0 + p < P) ? s_in[static_cast<int64_t>(n0 + n) * P + p0 + p] : 0.f;
     }
     __syncthreads();
-    for (int n = 0; n < SSM_L; ++n) {
-      const float sv = u_s[n][col];
-#pragma unroll
-      for (int r = 0; r < SSM_L / 4; ++r) y[r] += t_s[part + 4 * r][n] * sv;
-    }
+    for (int n = 0; n < SSM_L; n += 2)
+      y = __builtin_amdgcn_mfma_f32_32x32x2f32(t_s[ib + lane % 32][n + lane / 32], u_s[n + lane / 32][pb + lane % 32], y,
+                                               0, 0, 0);
   }
   __syncthreads();
   for (int i = threadIdx.x; i < SSM_L * 64; i += 256) {
@@ -275,14 +278,17 @@ ssm_chunk_outputs_kernel(const X* __restrict__ xbc, int64_t ld, const X* __restr
     t_s[j][p] = (j < rows && p0 + p < P) ? to_float(xbc[static_cast<int64_t>(first + j) * ld + head * P + p0 + p]) : 0.f;
   }
   __syncthreads();
+  // the chunk's own rows: sum_{j <= i} a[i][j] x_j[p]; rows j beyond the wave's last i have weight zero
+  ssm_floatx16 own = {};
+  for (int j = 0; j < ib + 32; j += 2)
+    own = __builtin_amdgcn_mfma_f32_32x32x2f32(a_s[ib + lane % 32][j + lane / 32], t_s[j + lane / 32][pb + lane % 32], own,
+                                               0, 0, 0);
   const float through = skip[head];
 #pragma unroll
-  for (int r = 0; r < SSM_L / 4; ++r) {
-    const int i = part + 4 * r;
-    float total = expf(l_s[i]) * y[r];
-    for (int j = 0; j <= i && j < rows; ++j) total += a_s[i][j] * t_s[j][col];
-    if (i < rows && p0 + col < P)
-      out[(static_cast<int64_t>(first + i) * H + head) * P + p0 + col] = total + through * t_s[i][col];
+  for (int v = 0; v < 16; ++v) {
+    const int i = ib + tile_row(v, lane), pc = pb + lane % 32;
+    if (i < rows && p0 + pc < P)
+      out[(static_cast<int64_t>(first + i) * H + head) * P + p0 + pc] = expf(l_s[i]) * y[v] + own[v] + through * t_s[i][pc];
   }
 }
 
@@ -407,7 +413,7 @@ extern "C" int distie_ssm_scan_chunked(const void* xbc, int dtype, int64_t ld, c
     ssm_chunk_sums_kernel<X><<<grid, 256, 0, stream>>>(static_cast<const X*>(xbc), ld, static_cast<const X*>(dt), ldd,
                                                       dt_bias, a_log, scratch, totals, static_cast<const int4*>(chunks),
                                                       H, P, N, G);
-    ssm_chunk_pairs_kernel<X><<<dim3(count, G, 4), 256, 0, stream>>>(static_cast<const X*>(xbc), ld, pairs,
+    ssm_chunk_pairs_kernel<X><<<dim3(count, G), 256, 0, stream>>>(static_cast<const X*>(xbc), ld, pairs,
                                                                     static_cast<const int4*>(chunks), H, P, N, G);
     ssm_chunk_states_kernel<<<dim3(B, H, parts), 256, 0, stream>>>(scratch, totals, state, first_chunk, state_slots, H, size);
     ssm_chunk_outputs_kernel<X><<<grid, 256, 0, stream>>>(static_cast<const X*>(xbc), ld, static_cast<const X*>(dt), ldd,

@@ -1662,7 +1662,8 @@ class HipOps(Ops):
             if vector.dtype != torch.float32 or tuple(vector.shape) != (H,):
                 raise KernelError("ssm_scan: dt_bias, a_log and skip are float32 [heads]")
         out = torch.empty((T, H * P), dtype=torch.float32, device=self.device)
-        if not self.captured and meta.host_cu_q is not None and meta.max_q >= self.SSM_CHUNKED_MIN_ROWS:
+        wide = N > self._ops.distie_ssm_scan_max_state()      # more rows a head than the row-by-row kernel keeps
+        if not self.captured and meta.host_cu_q is not None and (meta.max_q >= self.SSM_CHUNKED_MIN_ROWS or wide):
             count, packed, scratch = self._scan_chunks(meta, self._ops.distie_ssm_scan_chunk_rows(), H, N, P)
             key = ("ssm_totals", count, H, G)
             held = meta.scratch.get(key)
@@ -1678,8 +1679,9 @@ class HipOps(Ops):
                 self._stream()), "ssm_scan_chunked")
             _mark_written(state)
             return out
-        if N > self._ops.distie_ssm_scan_max_state():
-            raise KernelError(f"ssm_scan: a state of {N} rows a head is beyond the row-by-row kernel")
+        if wide:
+            raise KernelError(f"ssm_scan: a state of {N} rows a head is beyond the row-by-row kernel, which is all a "
+                              f"captured step can use")
         _check(self._ops.distie_ssm_scan(x_ptr, _code(xbc), ld, d_ptr, ldd, dt_bias.data_ptr(), a_log.data_ptr(),
                                          skip.data_ptr(), state.data_ptr(), out.data_ptr(), meta.cu_q.data_ptr(),
                                          meta.state_slots.data_ptr(), meta.num_requests, H, P, N, G, self._stream()),

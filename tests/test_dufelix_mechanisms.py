@@ -185,7 +185,7 @@ def test_state_space_mixer_alone(ops, sizes):
                LONG_CUTS, seed=1, slack=2.0)
 
 
-@pytest.mark.parametrize("H,P,N,G", [(3, 8, 4, 1), (4, 20, 12, 2), (2, 64, 64, 1), (2, 80, 130, 2)])
+@pytest.mark.parametrize("H,P,N,G", [(3, 8, 4, 1), (4, 20, 12, 2), (2, 64, 64, 1), (2, 80, 130, 2), (1, 24, 300, 1)])
 def test_state_space_scan_with_fast_and_slow_heads(ops, H, P, N, G):
     """The recurrence alone: step sizes from tiny to huge in one sequence (softplus far out on both sides), heads that
     forget at once beside heads that keep everything, over rows enough for several chunks, then row by row from the
