@@ -7,9 +7,10 @@ config.json names everything that can differ between models of the design:
     optionally, `weights_of`: another layer whose tensors (mixer, feed-forward, norms) this layer uses, with a cache
     or state of its own (its type and sizes are that layer's; an entry may repeat them).
 
-    attention mixer: heads, kv_heads, dim, vdim, rot {base, dims, scaling {factor, original, fast, slow}}, scale.
+    attention mixer: heads, kv_heads (heads if left out), dim, vdim (dim if left out), rot {base, dims, scaling {factor,
+    original, fast, slow}} (no rotation if left out, plain frequencies without `scaling`), scale.
     latent_attention mixer: heads, dim, rot_dim, vdim, kv_rank, q_rank, rot (as above, dims = rot_dim), scale.
-    mamba2 mixer: heads, vdim, state, groups, conv (taps), norm_groups.
+    mamba2 mixer: heads, vdim, state, groups, conv (taps), norm_groups (groups and norm_groups are one if left out).
 
 Tensors: `embed`, `head`, `final.norm`; layer i under `l<i>.`: `norm1`, `norm1b`, `norm2`, `norm2b`, `mix.*`,
 `mlp.gate|up|down`. Linear weights are [out, in]. Nothing here fixes a size. The one size a file may leave to a tensor's
@@ -91,10 +92,11 @@ class DufelixConfig:
                 continue                                         # (its sizes are the owner's, checked there)
             m = layer.get("mixer")
             if kind == "attention":
-                heads, kv_heads = _need(m, "heads", int, where), _need(m, "kv_heads", int, where)
+                heads = _need(m, "heads", int, where)
+                kv_heads = heads if m.get("kv_heads") is None else _need(m, "kv_heads", int, where)
                 if heads < 1 or kv_heads < 1 or heads % kv_heads:
                     raise ConfigError(f"{where}: heads must be a positive multiple of kv_heads")
-                if _need(m, "dim", int, where) < 1 or _need(m, "vdim", int, where) < 1:
+                if _need(m, "dim", int, where) < 1 or (m.get("vdim") is not None and _need(m, "vdim", int, where) < 1):
                     raise ConfigError(f"{where}: dim and vdim must be >= 1")
                 if not _need(m, "scale", float, where) > 0:
                     raise ConfigError(f"{where}: scale must be positive")
@@ -114,12 +116,15 @@ class DufelixConfig:
                 if int(m["rot"]["dims"]) != int(m["rot_dim"]):
                     raise ConfigError(f"{where}: rot.dims must equal rot_dim")
             else:
-                for key in ("heads", "vdim", "state", "groups", "conv", "norm_groups"):
+                for key in ("heads", "vdim", "state", "conv"):
                     if _need(m, key, int, where) < 1:
                         raise ConfigError(f"{where}: {key} must be >= 1")
-                if int(m["heads"]) % int(m["groups"]):
+                for key in ("groups", "norm_groups"):                      # one where a file leaves them out
+                    if m.get(key) is not None and _need(m, key, int, where) < 1:
+                        raise ConfigError(f"{where}: {key} must be >= 1")
+                if int(m["heads"]) % int(m.get("groups") or 1):
                     raise ConfigError(f"{where}: heads must be a multiple of groups")
-                if (int(m["heads"]) * int(m["vdim"])) % int(m["norm_groups"]):
+                if (int(m["heads"]) * int(m["vdim"])) % int(m.get("norm_groups") or 1):
                     raise ConfigError(f"{where}: heads * vdim must be a multiple of norm_groups")
             mlp = layer.get("mlp")
             if mlp is not None:
@@ -173,8 +178,8 @@ class DufelixConfig:
                                                 "scaling": rot.get("scaling")}) if rot else None
         if kind == "attention":
             return PartSpec("conv_gated_attention", base, {
-                "hidden_size": width, "num_heads": int(m["heads"]), "num_kv_heads": int(m["kv_heads"]),
-                "head_dim": int(m["dim"]), "value_dim": int(m["vdim"]), "conv_taps": 0, "window": None,
+                "hidden_size": width, "num_heads": int(m["heads"]), "num_kv_heads": int(m.get("kv_heads") or m["heads"]),
+                "head_dim": int(m["dim"]), "value_dim": int(m.get("vdim") or m["dim"]), "conv_taps": 0, "window": None,
                 "scale": float(m["scale"]), "output_gate": "head", "bias": False, "position": position})
         if kind == "latent_attention":
             if m.get("q_rank") is None:
@@ -187,8 +192,8 @@ class DufelixConfig:
                 "rotate": "neighbours", "position": position})
         return PartSpec("state_space_duality", base, {
             "hidden_size": width, "num_heads": int(m["heads"]), "value_dim": int(m["vdim"]),
-            "state_size": int(m["state"]), "groups": int(m["groups"]), "conv_taps": int(m["conv"]),
-            "norm_groups": int(m["norm_groups"]), "eps": eps})
+            "state_size": int(m["state"]), "groups": int(m.get("groups") or 1), "conv_taps": int(m["conv"]),
+            "norm_groups": int(m.get("norm_groups") or 1), "eps": eps})
 
     def model_spec(self) -> ModelSpec:
         data = self.data
