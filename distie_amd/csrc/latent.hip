@@ -310,6 +310,30 @@ __global__ void head_gate_kernel(const X* __restrict__ x, int ldh, int E, const 
   }
 }
 
+// bfloat16 with 16-byte loads and stores: eight of a head's columns a thread (E and ldh multiples of 8)
+__global__ void head_gate_bf16x8_kernel(const bf16_t* __restrict__ x, int ldh, int E, const bf16_t* __restrict__ gates,
+                                        int64_t ldg, bf16_t* __restrict__ out, int width, int T) {
+  const int per_row = width / 8;
+  const int64_t total = static_cast<int64_t>(T) * per_row;
+  for (int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; i < total;
+       i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+    const int64_t t = i / per_row;
+    const int c = 8 * static_cast<int>(i % per_row);
+    const int head = c / E, e = c % E;
+    const uint4 raw = *reinterpret_cast<const uint4*>(x + (t * (width / E) + head) * ldh + e);
+    const float g = sigmoidf(to_float(gates[t * ldg + head]));
+    const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+    uint32_t o[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const bf16_t lo = static_cast<bf16_t>(__uint_as_float(w[k] << 16) * g);
+      const bf16_t hi = static_cast<bf16_t>(__uint_as_float(w[k] & 0xffff0000u) * g);
+      o[k] = static_cast<uint32_t>(__builtin_bit_cast(uint16_t, lo)) | (static_cast<uint32_t>(__builtin_bit_cast(uint16_t, hi)) << 16);
+    }
+    *reinterpret_cast<uint4*>(out + t * width + c) = uint4{o[0], o[1], o[2], o[3]};
+  }
+}
+
 }  // namespace
 
 // the widest row (q_rank + kv_rank + rot_dim) that the kernel stages
@@ -415,6 +439,14 @@ extern "C" int distie_head_gate(const void* x, int x_dtype, int ldh, int E, cons
                                 void* out, int out_dtype, int T, int width, hipStream_t stream) {
   if (T <= 0) return 0;
   if (E < 1 || width < 1 || width % E || ldh < E || gates == nullptr || ldg < width / E) return DISTIE_BAD_ARGUMENT;
+  if (x_dtype == DISTIE_BF16 && g_dtype == DISTIE_BF16 && out_dtype == DISTIE_BF16 && E % 8 == 0 && ldh % 8 == 0 &&
+      reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0) {
+    const int64_t pieces = static_cast<int64_t>(T) * (width / 8);
+    const int blocks8 = static_cast<int>(pieces / 256 + 1 < 16384 ? pieces / 256 + 1 : 16384);
+    head_gate_bf16x8_kernel<<<blocks8, 256, 0, stream>>>(static_cast<const bf16_t*>(x), ldh, E,
+                                                         static_cast<const bf16_t*>(gates), ldg, static_cast<bf16_t*>(out), width, T);
+    return launch_status();
+  }
   const int threads = width >= 256 ? 256 : (width >= 128 ? 128 : 64);
   const dim3 grid(T, (width + threads - 1) / threads);
   DISTIE_DISPATCH(x_dtype, X, DISTIE_DISPATCH(g_dtype, G, DISTIE_DISPATCH(out_dtype, O,
