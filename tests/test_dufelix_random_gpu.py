@@ -48,18 +48,18 @@ def random_config(rng):
         vdim = rng.choice([4, 8, 10, 16, 24])
         parts = rng.choice([g for g in (1, 2, 3, 4) if (heads * vdim) % g == 0])
         return du.mamba(heads=heads, vdim=vdim, state=rng.choice([4, 8, 12, 16, 40]), groups=groups,
-                        conv=rng.choice([1, 2, 3, 4]), norm_groups=parts, mlp=mlp())
+                        conv=rng.choice([1, 2, 3, 4, 5]), norm_groups=parts, mlp=mlp())
 
     makers = [attention, latent, mamba]
     layers = [rng.choice(makers)() for _ in range(rng.randint(2, 5))]
     for i in range(len(layers)):
         if rng.random() < 0.5:
             layers.append(dict(layers[i], weights_of=i))
-    return du.make_config(layers, vocab=rng.choice([33, 50, 64]), width=rng.choice([24, 32, 40, 64]),
+    return du.make_config(layers, vocab=rng.choice([33, 50, 64]), width=rng.choice([24, 36, 40, 64]),
                           eps=rng.choice([1e-5, 1e-6]), embed_scale=rng.choice([1.0, 0.5, 6.0]))
 
 
-@pytest.mark.parametrize("seed", range(6))
+@pytest.mark.parametrize("seed", range(10))
 def test_random_models_and_traces(tmp_path, seed):
     rng = random.Random(1000 + seed)
     cfg = random_config(rng)
