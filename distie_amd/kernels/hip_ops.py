@@ -1646,6 +1646,9 @@ class HipOps(Ops):
     # ---- a state with one decay a head and token, attention over a shared latent (csrc/ssm.hip, csrc/latent.hip)
     SSM_CHUNKED_MIN_ROWS = 32        # a step with a portion of so many rows scans the state-space state in chunks
 
+    def ssm_scan_captures(self, state_size):
+        return state_size <= self._ops.distie_ssm_scan_max_state()
+
     def ssm_scan(self, xbc, dt, dt_bias, a_log, skip, state, meta, num_heads, value_dim, state_size, groups):
         xbc = self.dense(xbc)
         H, P, N, G = num_heads, value_dim, state_size, groups

@@ -286,6 +286,11 @@ class Ops(abc.ABC):
         leaves it. -> float32 [T, H * P]. Softplus, exponentials, the state, its products and sums in float32."""
         raise NotImplementedError(f"{type(self).__name__} has no state-space recurrence")
 
+    def ssm_scan_captures(self, state_size: int) -> bool:
+        """Whether `ssm_scan` at this state size can run inside a captured step (its launches then must not hang on the
+        step's row counts, which an implementation's kernel for large states may need)."""
+        return True
+
     def latent_norm_rope_write(self, down: torch.Tensor, q_rank: int, q_weight: Optional[torch.Tensor], kv_rank: int,
                                kv_weight: torch.Tensor, eps: float, rot_dim: int, inv_freq: Optional[torch.Tensor],
                                magnitude: float, neighbours: bool, meta: BatchMeta, group: int, k_cache: torch.Tensor,

@@ -71,6 +71,7 @@ class StateSpaceDuality(Mixer):
         self.out_weight = tensors["o"].contiguous()
 
     def prepare(self, ops) -> None:
+        self.capturable = bool(ops.ssm_scan_captures(self.state_size))
         ops.prepare_linear(self.in_weight, role="qkv")
         ops.prepare_linear(self.out_weight, role="attn_out")
 
