@@ -88,12 +88,12 @@ def prefixed(weights, prefix):
     return {k[len(prefix):]: v for k, v in weights.items() if k.startswith(prefix)}
 
 
-def mixer_case(ops, layer, spec_of, plain_of, lengths, cuts, width=40, seed=0, slack=1.0):
+def mixer_case(ops, layer, spec_of, plain_of, lengths, cuts, width=40, seed=0, slack=1.0, pages=64):
     cfg = du.make_config([layer], width=width)
     for dtype in act_types(ops):
         weights = du.random_weights(cfg, seed=seed, dtype=dtype)
         seqs = [rnd(n, width, seed=50 + i).to(dtype) for i, n in enumerate(lengths)]
-        got = run_mixer(ops, spec_of(cfg), prefixed(weights, "l0.mix."), seqs, cuts, dtype)
+        got = run_mixer(ops, spec_of(cfg), prefixed(weights, "l0.mix."), seqs, cuts, dtype, pages=pages)
         w = {k: v.to(F) for k, v in weights.items()}
         for i, s in enumerate(seqs):
             want = plain_of(s.to(F), w, "l0.mix.", layer["mixer"], torch.arange(len(s)), float(cfg["norm"]["eps"]))
@@ -121,6 +121,9 @@ def test_latent_attention_alone(ops, sizes):
                LENGTHS, CUTS, slack=2.0)
     mixer_case(ops, layer, dufelix_mixer, lambda h, w, p, m, pos, eps: plain.latent_attention(h, w, p, m, pos, eps),
                LONG_LENGTHS, LONG_CUTS, seed=1, slack=2.0)
+    # a portion long enough for the kernels that many rows choose
+    mixer_case(ops, layer, dufelix_mixer, lambda h, w, p, m, pos, eps: plain.latent_attention(h, w, p, m, pos, eps),
+               (300, 3), ((290, 1), (10, 2)), seed=2, slack=2.0, pages=128)
 
 
 def test_latent_cache_holds_the_latent_and_one_turned_part(ops):
@@ -280,8 +283,9 @@ def test_gated_activations_gates_by_head_and_scaled_embedding(ops):
 def test_products_by_head(ops):
     """Every head's own product, for few rows and for many, with inputs and results that lie apart in wider rows."""
     dev = lambda t: t.to(ops.device)
-    for T in (1, 5, 16, 17, 150):
-        for H, N, K, lx, lo in ((3, 24, 12, 20, 32), (1, 16, 16, 16, 16), (5, 18, 10, 16, 24), (4, 72, 104, 128, 72)):
+    for T in (1, 5, 16, 17, 150, 300):
+        for H, N, K, lx, lo in ((3, 24, 12, 20, 32), (1, 16, 16, 16, 16), (5, 18, 10, 16, 24), (4, 72, 104, 128, 72),
+                                (2, 40, 200, 208, 48), (3, 100, 128, 160, 112)):
             for dtype in act_types(ops):
                 x, w = rnd(T, H * lx, seed=1).to(dtype), rnd(H, N, K, seed=2, scale=0.3).to(dtype)
                 got = ops.heads_linear(dev(x), dev(w), lx, lo).float().cpu().view(T, H, lo)
